@@ -1,0 +1,238 @@
+"""ctypes view of the device library's C ABI (include/compressgnn_abi.h).
+
+torch tensors supply device memory and the current stream; every computation goes
+through libcgnn_hip.so.  There is no fallback: if the library is missing or a call
+fails, an exception is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcgnn_hip.so")
+
+F32, F64 = 0, 1
+SPMM_AUTO, SPMM_ROW, SPMM_NNZ = 0, 1, 2
+
+EXPORTS = [
+    "cgnn_last_error", "cgnn_version",
+    "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_pair",
+    "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
+    "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_hash", "cgnn_lsh_scan", "cgnn_lsh_finish",
+    "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
+    "cgnn_cluster_mean_workspace_bytes", "cgnn_cluster_mean", "cgnn_cluster_mean_backward",
+    "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_copy_bytes",
+]
+
+
+class CsrStruct(ctypes.Structure):
+    _fields_ = [
+        ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("nnz", ctypes.c_int64),
+        ("rowptr", ctypes.c_void_p), ("colidx", ctypes.c_void_p), ("rowidx", ctypes.c_void_p),
+        ("val", ctypes.c_void_p), ("max_row_nnz", ctypes.c_int32), ("seg_nnz", ctypes.c_int32),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libcgnn_hip.so is not built (%s); run `python -m compressgnn_amd.build hip`" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        L.cgnn_last_error.restype = ctypes.c_char_p
+        L.cgnn_version.restype = ctypes.c_char_p
+        for name in ("cgnn_spmm_workspace_bytes", "cgnn_lsh_scan_workspace_bytes",
+                     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes"):
+            getattr(L, name).restype = ctypes.c_size_t
+        _lib = L
+    return _lib
+
+
+class CgnnError(RuntimeError):
+    pass
+
+
+def check(rc):
+    if rc != 0:
+        raise CgnnError("cgnn error %d: %s" % (rc, lib().cgnn_last_error().decode()))
+
+
+def dtype_code(dtype):
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.float64:
+        return F64
+    raise TypeError("only float32 and float64 are supported, got %s" % dtype)
+
+
+def ptr(t):
+    return ctypes.c_void_p(0 if t is None or t.numel() == 0 and t.data_ptr() == 0 else t.data_ptr())
+
+
+def stream_of(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def i64(x):
+    return ctypes.c_int64(int(x))
+
+
+class DeviceCsr:
+    """A CSR block on the device with int32 indices (the layout the kernels read)."""
+
+    def __init__(self, rows, cols, rowptr, colidx, val, rowidx=None, max_row_nnz=0, seg_nnz=0):
+        self.rows, self.cols = int(rows), int(cols)
+        self.rowptr, self.colidx, self.val, self.rowidx = rowptr, colidx, val, rowidx
+        self.nnz = int(colidx.numel())
+        self.max_row_nnz, self.seg_nnz = int(max_row_nnz), int(seg_nnz)
+        self._ws = {}
+
+    @classmethod
+    def from_host(cls, rows, cols, rowptr, colidx, val, device, with_rowidx=True, seg_nnz=0):
+        """rowptr/colidx: integer arrays or tensors on the host; val: float tensor/array or None."""
+        rp = torch.as_tensor(rowptr).to(torch.int64)
+        ci = torch.as_tensor(colidx).to(torch.int64)
+        lens = rp[1:] - rp[:-1]
+        max_row = int(lens.max()) if lens.numel() else 0
+        rowidx = None
+        if with_rowidx:
+            rowidx = torch.repeat_interleave(torch.arange(rows, dtype=torch.int32), lens).to(device)
+        v = None if val is None else torch.as_tensor(val).to(device)
+        return cls(rows, cols, rp.to(torch.int32).to(device), ci.to(torch.int32).to(device), v, rowidx,
+                   max_row, seg_nnz)
+
+    def struct(self):
+        s = CsrStruct()
+        s.rows, s.cols, s.nnz = self.rows, self.cols, self.nnz
+        s.rowptr = self.rowptr.data_ptr()
+        s.colidx = self.colidx.data_ptr() if self.nnz else 0
+        s.rowidx = self.rowidx.data_ptr() if (self.rowidx is not None and self.nnz) else 0
+        s.val = self.val.data_ptr() if (self.val is not None and self.nnz) else 0
+        s.max_row_nnz, s.seg_nnz = self.max_row_nnz, self.seg_nnz
+        return s
+
+    def workspace(self, F, dtype, kernel):
+        """Scratch for one (F, dtype, kernel), cached on the block (per stream use is the
+        caller's business: calls on one stream are ordered)."""
+        s = self.struct()
+        need = lib().cgnn_spmm_workspace_bytes(ctypes.byref(s), i64(F), dtype_code(dtype), kernel)
+        key = (int(F), dtype, kernel)
+        ws = self._ws.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=self.rowptr.device)
+            self._ws[key] = ws
+        return ws, need
+
+
+def spmm(A, X, Y=None, accumulate=False, kernel=SPMM_AUTO):
+    """Y (+)= A @ X through cgnn_spmm.  Returns Y (allocated when None)."""
+    F = X.shape[1]
+    if Y is None:
+        Y = torch.empty((A.rows, F), dtype=X.dtype, device=X.device)
+        accumulate = False
+    ws, need = A.workspace(F, X.dtype, kernel)
+    s = A.struct()
+    check(lib().cgnn_spmm(ctypes.byref(s), dtype_code(X.dtype), ptr(X), ptr(Y), i64(F),
+                          ctypes.c_int(1 if accumulate else 0), ctypes.c_int(kernel), ptr(ws),
+                          ctypes.c_size_t(need), stream_of(X)))
+    return Y
+
+
+def spmm_pair(A0, X0, A1, X1, Y=None):
+    F = X0.shape[1]
+    if Y is None:
+        Y = torch.empty((A0.rows, F), dtype=X0.dtype, device=X0.device)
+    s0, s1 = A0.struct(), A1.struct()
+    check(lib().cgnn_spmm_pair(ctypes.byref(s0), ptr(X0), ctypes.byref(s1), ptr(X1),
+                               dtype_code(X0.dtype), ptr(Y), i64(F), stream_of(X0)))
+    return Y
+
+
+def lsh_assign(x, planes, bits):
+    """(ids int64 [N], counts int32 [active+1], active) through the three LSH entry
+    points; one host read of the active-bucket count."""
+    N, F = x.shape
+    dev = x.device
+    L = lib()
+    buckets = 1 << bits
+    bucket_count = torch.empty(buckets, dtype=torch.int32, device=dev)
+    prefix = torch.empty(buckets, dtype=torch.int32, device=dev)
+    scan_bytes = L.cgnn_lsh_scan_workspace_bytes(bits)
+    scan_ws = torch.empty(max(scan_bytes, 1), dtype=torch.uint8, device=dev)
+    raw = torch.empty(N, dtype=torch.int32, device=dev)
+    ids = torch.empty(N, dtype=torch.int64, device=dev)
+    st = stream_of(x)
+    check(L.cgnn_lsh_hash(i64(N), i64(F), bits, dtype_code(x.dtype), ptr(x), ptr(planes), ptr(raw),
+                          ptr(bucket_count), st))
+    check(L.cgnn_lsh_scan(bits, ptr(bucket_count), ptr(prefix), ptr(scan_ws), ctypes.c_size_t(scan_bytes), st))
+    active = int(prefix[-1].item())
+    counts = torch.zeros(active + 1, dtype=torch.int32, device=dev)
+    check(L.cgnn_lsh_finish(i64(N), bits, ptr(raw), ptr(bucket_count), ptr(prefix), ptr(ids), ptr(counts), st))
+    return ids, counts, active
+
+
+def cluster_members(ids, groups):
+    """(offsets int32 [groups+1], perm int32 [N], sorted_id int32 [N])."""
+    N = ids.numel()
+    dev = ids.device
+    L = lib()
+    offsets = torch.empty(groups + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(N, dtype=torch.int32, device=dev)
+    sorted_id = torch.empty(N, dtype=torch.int32, device=dev)
+    need = L.cgnn_cluster_members_workspace_bytes(i64(N), i64(groups))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    check(L.cgnn_cluster_members(i64(N), i64(groups), ptr(ids), ptr(offsets), ptr(perm), ptr(sorted_id),
+                                 ptr(ws), ctypes.c_size_t(need), stream_of(ids)))
+    return offsets, perm, sorted_id
+
+
+def cluster_mean(x, members, counts):
+    offsets, perm, sorted_id = members
+    N, F = x.shape
+    groups = counts.numel()
+    L = lib()
+    reps = torch.empty((groups, F), dtype=x.dtype, device=x.device)
+    need = L.cgnn_cluster_mean_workspace_bytes(i64(N), i64(F), i64(groups), dtype_code(x.dtype))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    check(L.cgnn_cluster_mean(i64(N), i64(F), i64(groups), dtype_code(x.dtype), ptr(x), ptr(offsets),
+                              ptr(perm), ptr(sorted_id), ptr(counts), ptr(reps), ptr(ws),
+                              ctypes.c_size_t(need), stream_of(x)))
+    return reps
+
+
+def cluster_mean_backward(grad, ids, counts):
+    N = ids.numel()
+    F = grad.shape[1]
+    dx = torch.empty((N, F), dtype=grad.dtype, device=grad.device)
+    check(lib().cgnn_cluster_mean_backward(i64(N), i64(F), i64(counts.numel()), dtype_code(grad.dtype),
+                                           ptr(grad), ptr(ids), ptr(counts), ptr(dx), stream_of(grad)))
+    return dx
+
+
+def reconstruct(reps, ids, bias=None, relu=False):
+    N = ids.numel()
+    F = reps.shape[1]
+    out = torch.empty((N, F), dtype=reps.dtype, device=reps.device)
+    check(lib().cgnn_reconstruct(i64(N), i64(F), i64(reps.shape[0]), dtype_code(reps.dtype), ptr(reps),
+                                 ptr(ids), ptr(bias), ctypes.c_int(1 if relu else 0), ptr(out),
+                                 stream_of(reps)))
+    return out
+
+
+def reconstruct_backward(grad, output, members, groups, relu=False):
+    offsets, perm, sorted_id = members
+    N, F = grad.shape
+    L = lib()
+    reps_grad = torch.empty((groups, F), dtype=grad.dtype, device=grad.device)
+    need = L.cgnn_cluster_mean_workspace_bytes(i64(N), i64(F), i64(groups), dtype_code(grad.dtype))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=grad.device)
+    check(L.cgnn_reconstruct_backward(i64(N), i64(F), i64(groups), dtype_code(grad.dtype), ptr(grad),
+                                      ptr(output), ptr(offsets), ptr(perm), ptr(sorted_id),
+                                      ctypes.c_int(1 if relu else 0), ptr(reps_grad), ptr(ws),
+                                      ctypes.c_size_t(need), stream_of(grad)))
+    return reps_grad

@@ -1,0 +1,561 @@
+// Transformation-compression kernels for gfx950: LSH projection + sign hash + bucket
+// histogram, occupancy scan, id remap, row gathers (mean backward, reconstruct with
+// fused bias + ReLU).  The per-cluster sums (mean forward, reconstruct backward) run
+// on the member lists through the nnz-schedule SpMM in spmm.hip.
+#include "common.h"
+
+namespace cgnn {
+
+int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, void *Y, int64_t F,
+                 bool relu_mask, void *ws, size_t ws_bytes, hipStream_t stream);
+
+namespace {
+
+// ------------------------------------------------------------------ LSH hash ---
+//
+// One lane per row, one wave (64 rows) per workgroup.  The wave stages its 64 rows
+// of X, KS columns at a time, in LDS with fully coalesced 16-byte loads, then every
+// lane walks its own row: h_j = fma(x_k, W[k,j], h_j) for k ascending, which fixes
+// the rounding of every projection (the CPU oracle uses the same chain).  W is read
+// with wave-uniform addresses, i.e. through the scalar unit, so the inner loop is one
+// LDS read per 4 k and HB vector FMAs per k.  The LDS row stride is odd in units of
+// the access width, which keeps the 64 strided row reads free of bank conflicts.
+//
+// HB = number of accumulators (bits rounded up); columns >= bits repeat the last
+// real column and are ignored when the code is formed.
+
+constexpr int kLshRows = 64;
+constexpr int kLshMaxSlab = 128;  // columns staged per pass (floats)
+
+template <typename T>
+struct LshArgs {
+    const T *__restrict__ X;
+    const T *__restrict__ W;
+    int32_t *raw_code;
+    int32_t *bucket_count;
+    int64_t N;
+    int32_t F;
+    int32_t bits;
+    int32_t slab;      // columns per pass, multiple of VEC
+    int32_t stride_v;  // LDS row stride in units of VEC elements (odd)
+    uint32_t magic;    // floor(2^32 / slab_v) + 1: i / slab_v == mulhi(i, magic) for i < 2^16
+};
+
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) LPack {
+    T v[VEC];
+};
+
+template <typename T, int VEC, int HB, bool EXACT>
+__global__ __launch_bounds__(kLshRows) void lsh_hash_kernel(LshArgs<T> a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    LPack<T, VEC> *tile = reinterpret_cast<LPack<T, VEC> *>(lds_raw);
+    const int lane = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * kLshRows;
+    const int rows_here = (int)min((int64_t)kLshRows, a.N - row0);
+    const int H = a.bits;
+    T acc[HB];
+#pragma unroll
+    for (int j = 0; j < HB; ++j) acc[j] = T(0);
+
+    for (int k0 = 0; k0 < a.F; k0 += a.slab) {
+        const int ks = min(a.slab, a.F - k0);  // multiple of VEC
+        const int ks_v = ks / VEC;
+        // magic division is exact for the full slab; a shorter last slab divides directly
+        const bool full = ks == a.slab;
+        const int total = rows_here * ks_v;
+        __syncthreads();
+        for (int i = lane; i < total; i += kLshRows) {
+            int r = full ? (int)__umulhi((uint32_t)i, a.magic) : i / ks_v;
+            int c = i - r * ks_v;
+            const T *src = a.X + (row0 + r) * (int64_t)a.F + k0 + c * VEC;
+            tile[r * a.stride_v + c] = *reinterpret_cast<const LPack<T, VEC> *>(src);
+        }
+        __syncthreads();
+        if (lane < rows_here) {
+            const LPack<T, VEC> *mine = tile + lane * a.stride_v;
+            for (int c = 0; c < ks_v; ++c) {
+                LPack<T, VEC> x = mine[c];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const int k = k0 + c * VEC + i;
+                    const T *wrow = a.W + (int64_t)k * (EXACT ? HB : H);
+#pragma unroll
+                    for (int j = 0; j < HB; ++j) {
+                        T w = EXACT ? wrow[j] : wrow[min(j, H - 1)];
+                        acc[j] = __builtin_fma(x.v[i], w, acc[j]);
+                    }
+                }
+            }
+        }
+    }
+    if (lane < rows_here) {
+        int code = 0;
+#pragma unroll
+        for (int j = 0; j < HB; ++j)
+            if (j < H) code = (code << 1) | (acc[j] > T(0) ? 1 : 0);
+        a.raw_code[row0 + lane] = code;
+        atomicAdd(a.bucket_count + code, 1);
+    }
+}
+
+// bits == 0 or F == 0: every projection is empty, code 0.
+__global__ void lsh_trivial_kernel(int32_t *raw_code, int32_t *bucket_count, int64_t N) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < N) raw_code[i] = 0;
+    if (i == 0) bucket_count[0] = (int32_t)N;
+}
+
+__global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = v;
+}
+
+int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t stream) {
+    if (n == 0) return CGNN_OK;
+    int64_t blocks = ceil_div(n, kBlock);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, p, n, v);
+    return check_launch("fill");
+}
+
+template <typename T, int VEC, int HB, bool EXACT>
+int launch_lsh(const LshArgs<T> &a, hipStream_t stream) {
+    const size_t lds = (size_t)kLshRows * a.stride_v * VEC * sizeof(T);
+    const int64_t blocks = ceil_div(a.N, kLshRows);
+    hipLaunchKernelGGL((lsh_hash_kernel<T, VEC, HB, EXACT>), dim3((unsigned)blocks), dim3(kLshRows),
+                       lds, stream, a);
+    return check_launch("lsh_hash");
+}
+
+template <typename T, int VEC>
+int dispatch_lsh(const LshArgs<T> &a, hipStream_t stream) {
+    const int H = a.bits;
+    if (H == 8) return launch_lsh<T, VEC, 8, true>(a, stream);
+    if (H == 16) return launch_lsh<T, VEC, 16, true>(a, stream);
+    if (H < 8) return launch_lsh<T, VEC, 8, false>(a, stream);
+    if (H < 16) return launch_lsh<T, VEC, 16, false>(a, stream);
+    return launch_lsh<T, VEC, 32, false>(a, stream);
+}
+
+template <typename T>
+int lsh_hash_typed(int64_t N, int64_t F, int bits, const void *X, const void *W, int32_t *raw_code,
+                   int32_t *bucket_count, hipStream_t stream) {
+    LshArgs<T> a{};
+    a.X = static_cast<const T *>(X);
+    a.W = static_cast<const T *>(W);
+    a.raw_code = raw_code;
+    a.bucket_count = bucket_count;
+    a.N = N;
+    a.F = (int32_t)F;
+    a.bits = bits;
+    constexpr int WIDE = 16 / sizeof(T);  // elements per 16-byte access
+    const bool wide = (F % WIDE == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0);
+    const int vec = wide ? WIDE : 1;
+    const int max_slab = kLshMaxSlab * 4 / (int)sizeof(T);
+    int slab = (int)(F < max_slab ? F : max_slab);
+    slab -= slab % vec;
+    a.slab = slab;
+    const int slab_v = slab / vec;
+    a.stride_v = slab_v | 1;
+    a.magic = (uint32_t)((1ull << 32) / (uint32_t)slab_v) + 1u;
+    if (wide) return dispatch_lsh<T, WIDE>(a, stream);
+    return dispatch_lsh<T, 1>(a, stream);
+}
+
+// ---------------------------------------------------------- occupancy scan -----
+//
+// prefix[b] = #{b' <= b : bucket_count[b'] != 0}.  Three passes over tiles of
+// kScanTile buckets: tile totals, an in-place exclusive scan of the totals by one
+// workgroup, then the tile scans offset by their totals.
+
+constexpr int kScanItems = 16;
+constexpr int kScanTile = kBlock * kScanItems;
+
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        int n = __shfl_up(v, d, kWave);
+        if ((int)(threadIdx.x % kWave) >= d) v += n;
+    }
+    return v;
+}
+
+// Inclusive scan of one value per thread over the workgroup; returns the inclusive
+// value and the workgroup total.
+__device__ __forceinline__ int block_inclusive_scan(int v, int *total) {
+    __shared__ int wave_sum[kBlock / kWave];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    int inc = wave_inclusive_scan(v);
+    __syncthreads();  // wave_sum may still be read by a previous call
+    if (lane == kWave - 1) wave_sum[wave] = inc;
+    __syncthreads();
+    int offset = 0, sum = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w) {
+        if (w < wave) offset += wave_sum[w];
+        sum += wave_sum[w];
+    }
+    *total = sum;
+    return inc + offset;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_tile_totals_kernel(const int32_t *count, int64_t n,
+                                                                 int32_t *totals) {
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i)
+        if (base + i < n) s += count[base + i] != 0;
+    int total;
+    block_inclusive_scan(s, &total);
+    if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_totals_kernel(int32_t *totals, int64_t m) {
+    int running = 0;
+    for (int64_t base = 0; base < m; base += kBlock) {
+        int64_t i = base + threadIdx.x;
+        int v = i < m ? totals[i] : 0;
+        int total;
+        int inc = block_inclusive_scan(v, &total);
+        if (i < m) totals[i] = running + inc - v;  // exclusive
+        running += total;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void scan_apply_kernel(const int32_t *count, int64_t n,
+                                                           const int32_t *totals, int32_t *prefix) {
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    int flag[kScanItems];
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+        flag[i] = (base + i < n) ? (count[base + i] != 0) : 0;
+        s += flag[i];
+    }
+    int total;
+    int inc = block_inclusive_scan(s, &total);
+    int run = totals[blockIdx.x] + inc - s;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+        run += flag[i];
+        if (base + i < n) prefix[base + i] = run;
+    }
+}
+
+__global__ void lsh_finish_kernel(int64_t N, int64_t buckets, const int32_t *raw_code,
+                                  const int32_t *bucket_count, const int32_t *prefix, int64_t *ids,
+                                  int32_t *counts) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N || i < buckets;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        if (i < N) ids[i] = prefix[raw_code[i]];
+        if (i < buckets) {
+            int c = bucket_count[i];
+            if (c) counts[prefix[i]] = c;
+        }
+    }
+}
+
+// ------------------------------------------------------------ row gathers ------
+//
+// out[i,:] = f(src[ids[i],:]) with LPR lanes per row and VEC features per lane; each
+// lane group handles kGatherRows consecutive rows with all loads issued first.
+
+constexpr int kGatherRows = 4;
+enum { GATHER_MEAN_GRAD = 0, GATHER_RECONSTRUCT = 1 };
+
+template <typename T>
+struct GatherArgs {
+    const T *__restrict__ src;       // [groups x F]
+    const int64_t *__restrict__ ids; // [N]
+    const int32_t *__restrict__ counts;
+    const T *__restrict__ bias;
+    T *__restrict__ out;             // [N x F]
+    int64_t N, F, groups;
+    int32_t relu;
+};
+
+template <typename T, int VEC, int LPR, int OP>
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
+    constexpr int GPB = kBlock / LPR;
+    const int lane = threadIdx.x % LPR;
+    int64_t first = ((int64_t)blockIdx.x * GPB + threadIdx.x / LPR) * kGatherRows;
+    if (first >= a.N) return;
+    int64_t g[kGatherRows];
+#pragma unroll
+    for (int r = 0; r < kGatherRows; ++r) {
+        int64_t i = first + r < a.N ? first + r : a.N - 1;
+        g[r] = a.ids[i];
+    }
+    T denom[kGatherRows];
+    if constexpr (OP == GATHER_MEAN_GRAD) {
+#pragma unroll
+        for (int r = 0; r < kGatherRows; ++r) denom[r] = (T)max(a.counts[g[r]], 1);
+    }
+    for (int64_t f = (int64_t)lane * VEC; f < a.F; f += (int64_t)LPR * VEC) {
+        LPack<T, VEC> x[kGatherRows];
+#pragma unroll
+        for (int r = 0; r < kGatherRows; ++r)
+            x[r] = *reinterpret_cast<const LPack<T, VEC> *>(a.src + g[r] * a.F + f);
+        LPack<T, VEC> b;
+        if constexpr (OP == GATHER_RECONSTRUCT) {
+            if (a.bias) b = *reinterpret_cast<const LPack<T, VEC> *>(a.bias + f);
+        }
+#pragma unroll
+        for (int r = 0; r < kGatherRows; ++r) {
+            if (first + r >= a.N) break;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                T v = x[r].v[i];
+                if constexpr (OP == GATHER_MEAN_GRAD) {
+                    v = v / denom[r];
+                } else {
+                    if (a.bias) v = v + b.v[i];
+                    v = (a.relu && v < T(0)) ? T(0) : v;
+                }
+                x[r].v[i] = v;
+            }
+            *reinterpret_cast<LPack<T, VEC> *>(a.out + (first + r) * a.F + f) = x[r];
+        }
+    }
+}
+
+template <typename T, int VEC, int OP>
+int launch_gather_lpr(const GatherArgs<T> &a, hipStream_t stream) {
+    const int64_t slots = a.F / VEC;
+    int lpr = pow2_ceil(slots);
+    lpr = lpr <= 4 ? 4 : (lpr <= 8 ? 8 : (lpr <= 16 ? 16 : (lpr <= 32 ? 32 : 64)));
+    const int gpb = kBlock / lpr;
+    const int64_t groups_needed = ceil_div(a.N, kGatherRows);
+    dim3 grid((unsigned)ceil_div(groups_needed, gpb)), block(kBlock);
+    switch (lpr) {
+        case 4: hipLaunchKernelGGL((gather_rows_kernel<T, VEC, 4, OP>), grid, block, 0, stream, a); break;
+        case 8: hipLaunchKernelGGL((gather_rows_kernel<T, VEC, 8, OP>), grid, block, 0, stream, a); break;
+        case 16: hipLaunchKernelGGL((gather_rows_kernel<T, VEC, 16, OP>), grid, block, 0, stream, a); break;
+        case 32: hipLaunchKernelGGL((gather_rows_kernel<T, VEC, 32, OP>), grid, block, 0, stream, a); break;
+        default: hipLaunchKernelGGL((gather_rows_kernel<T, VEC, 64, OP>), grid, block, 0, stream, a); break;
+    }
+    return check_launch("gather_rows");
+}
+
+template <typename T, int OP>
+int launch_gather(const GatherArgs<T> &a, hipStream_t stream) {
+    if (a.N == 0 || a.F == 0) return CGNN_OK;
+    if (ceil_div(a.N, kGatherRows) >= ((int64_t)1 << 31))
+        return fail(CGNN_EUNSUPPORTED, "gather: too many rows");
+    constexpr int WIDE = 16 / sizeof(T);
+    auto al = [](const void *p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (a.F % WIDE == 0 && al(a.src) && al(a.out) && al(a.bias)) return launch_gather_lpr<T, WIDE, OP>(a, stream);
+    return launch_gather_lpr<T, 1, OP>(a, stream);
+}
+
+template <typename T>
+__global__ void divide_counts_kernel(T *reps, const int32_t *counts, int64_t groups, int64_t F) {
+    const int64_t n = groups * F;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        int c = counts[i / F];
+        reps[i] = reps[i] / (T)max(c, 1);
+    }
+}
+
+__global__ void copy16_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+int check_bits(int bits) {
+    if (bits < 0 || bits > 30) return fail(CGNN_EINVAL, "hash bits must be in [0,30]");
+    return CGNN_OK;
+}
+
+size_t scan_tiles(int bits) { return (size_t)ceil_div((int64_t)1 << bits, kScanTile); }
+
+cgnn_csr members_csr(int64_t N, int64_t groups, const int32_t *offsets, const int32_t *perm,
+                     const int32_t *sorted_id) {
+    cgnn_csr A{};
+    A.rows = groups;
+    A.cols = N;
+    A.nnz = N;
+    A.rowptr = offsets;
+    A.colidx = perm;
+    A.rowidx = sorted_id;
+    A.val = nullptr;
+    A.max_row_nnz = 0;
+    A.seg_nnz = 0;
+    return A;
+}
+
+}  // namespace
+}  // namespace cgnn
+
+using namespace cgnn;
+
+extern "C" int cgnn_lsh_hash(int64_t N, int64_t F, int bits, int dtype, const void *X, const void *W,
+                             int32_t *raw_code, int32_t *bucket_count, cgnn_stream_t stream) {
+    int rc = check_bits(bits);
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(N >= 0 && F >= 0, "cgnn_lsh_hash: negative size");
+    CGNN_REQUIRE(N < INT32_MAX, "cgnn_lsh_hash: row count exceeds the int32 bucket counters");
+    CGNN_REQUIRE(F < (1 << 24), "cgnn_lsh_hash: feature width too large");
+    CGNN_REQUIRE(bucket_count != nullptr, "cgnn_lsh_hash: bucket_count is null");
+    CGNN_REQUIRE(N == 0 || raw_code != nullptr, "cgnn_lsh_hash: raw_code is null");
+    rc = fill_i32(bucket_count, (int64_t)1 << bits, 0, stream);
+    if (rc != CGNN_OK || N == 0) return rc;
+    if (bits == 0 || F == 0) {
+        hipLaunchKernelGGL(lsh_trivial_kernel, dim3((unsigned)ceil_div(N, kBlock)), dim3(kBlock), 0,
+                           stream, raw_code, bucket_count, N);
+        return check_launch("lsh_trivial");
+    }
+    CGNN_REQUIRE(X != nullptr && W != nullptr, "cgnn_lsh_hash: X or W is null");
+    if (dtype == CGNN_F32) return lsh_hash_typed<float>(N, F, bits, X, W, raw_code, bucket_count, stream);
+    if (dtype == CGNN_F64) return lsh_hash_typed<double>(N, F, bits, X, W, raw_code, bucket_count, stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_lsh_hash: dtype must be f32 or f64");
+}
+
+extern "C" size_t cgnn_lsh_scan_workspace_bytes(int bits) {
+    if (bits < 0 || bits > 30) return 0;
+    return align_up(scan_tiles(bits) * sizeof(int32_t), 256);
+}
+
+extern "C" int cgnn_lsh_scan(int bits, const int32_t *bucket_count, int32_t *prefix, void *workspace,
+                             size_t workspace_bytes, cgnn_stream_t stream) {
+    int rc = check_bits(bits);
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(bucket_count != nullptr && prefix != nullptr, "cgnn_lsh_scan: null array");
+    if (workspace == nullptr || workspace_bytes < cgnn_lsh_scan_workspace_bytes(bits))
+        return fail(CGNN_EWORKSPACE, "cgnn_lsh_scan: workspace too small");
+    const int64_t n = (int64_t)1 << bits;
+    const int64_t tiles = (int64_t)scan_tiles(bits);
+    int32_t *totals = static_cast<int32_t *>(workspace);
+    hipLaunchKernelGGL(scan_tile_totals_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream,
+                       bucket_count, n, totals);
+    hipLaunchKernelGGL(scan_totals_kernel, dim3(1), dim3(kBlock), 0, stream, totals, tiles);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, bucket_count,
+                       n, totals, prefix);
+    return check_launch("lsh_scan");
+}
+
+extern "C" int cgnn_lsh_finish(int64_t N, int bits, const int32_t *raw_code,
+                               const int32_t *bucket_count, const int32_t *prefix, int64_t *ids,
+                               int32_t *counts, cgnn_stream_t stream) {
+    int rc = check_bits(bits);
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(N >= 0, "cgnn_lsh_finish: negative size");
+    CGNN_REQUIRE(bucket_count && prefix && counts, "cgnn_lsh_finish: null array");
+    CGNN_REQUIRE(N == 0 || (raw_code && ids), "cgnn_lsh_finish: null array");
+    const int64_t buckets = (int64_t)1 << bits;
+    int64_t work = N > buckets ? N : buckets;
+    int64_t blocks = ceil_div(work, kBlock);
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(lsh_finish_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, N, buckets,
+                       raw_code, bucket_count, prefix, ids, counts);
+    return check_launch("lsh_finish");
+}
+
+extern "C" size_t cgnn_cluster_mean_workspace_bytes(int64_t N, int64_t F, int64_t groups, int dtype) {
+    cgnn_csr A = members_csr(N, groups, nullptr, nullptr, nullptr);
+    return cgnn_spmm_workspace_bytes(&A, F, dtype, CGNN_SPMM_NNZ);
+}
+
+template <typename T>
+static int divide_counts(void *reps, const int32_t *counts, int64_t groups, int64_t F,
+                         hipStream_t stream) {
+    const int64_t n = groups * F;
+    if (n == 0) return CGNN_OK;
+    int64_t blocks = ceil_div(n, kBlock);
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(divide_counts_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                       static_cast<T *>(reps), counts, groups, F);
+    return check_launch("divide_counts");
+}
+
+extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype, const void *X,
+                                 const int32_t *offsets, const int32_t *perm,
+                                 const int32_t *sorted_id, const int32_t *counts, void *reps,
+                                 void *workspace, size_t workspace_bytes, cgnn_stream_t stream) {
+    CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 1, "cgnn_cluster_mean: bad size");
+    CGNN_REQUIRE(dtype == CGNN_F32 || dtype == CGNN_F64, "cgnn_cluster_mean: dtype must be f32 or f64");
+    if (F == 0) return CGNN_OK;
+    CGNN_REQUIRE(offsets && counts && reps, "cgnn_cluster_mean: null array");
+    CGNN_REQUIRE(N == 0 || (X && perm && sorted_id), "cgnn_cluster_mean: null array");
+    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id);
+    int rc = spmm_members(&A, dtype, X, nullptr, reps, F, false, workspace, workspace_bytes, stream);
+    if (rc != CGNN_OK) return rc;
+    if (dtype == CGNN_F32) return divide_counts<float>(reps, counts, groups, F, stream);
+    return divide_counts<double>(reps, counts, groups, F, stream);
+}
+
+template <typename T, int OP>
+static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, const int64_t *ids,
+                        const int32_t *counts, const void *bias, int relu, void *out,
+                        hipStream_t stream) {
+    GatherArgs<T> a{};
+    a.src = static_cast<const T *>(src);
+    a.ids = ids;
+    a.counts = counts;
+    a.bias = static_cast<const T *>(bias);
+    a.out = static_cast<T *>(out);
+    a.N = N;
+    a.F = F;
+    a.groups = groups;
+    a.relu = relu ? 1 : 0;
+    return launch_gather<T, OP>(a, stream);
+}
+
+extern "C" int cgnn_cluster_mean_backward(int64_t N, int64_t F, int64_t groups, int dtype,
+                                          const void *grad, const int64_t *ids,
+                                          const int32_t *counts, void *dx, cgnn_stream_t stream) {
+    CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 1, "cgnn_cluster_mean_backward: bad size");
+    if (N == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(grad && ids && counts && dx, "cgnn_cluster_mean_backward: null array");
+    if (dtype == CGNN_F32)
+        return gather_typed<float, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, nullptr, 0, dx, stream);
+    if (dtype == CGNN_F64)
+        return gather_typed<double, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, nullptr, 0, dx, stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_cluster_mean_backward: dtype must be f32 or f64");
+}
+
+extern "C" int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
+                                const int64_t *ids, const void *bias, int relu, void *out,
+                                cgnn_stream_t stream) {
+    CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 0, "cgnn_reconstruct: bad size");
+    if (N == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(reps && ids && out, "cgnn_reconstruct: null array");
+    if (dtype == CGNN_F32)
+        return gather_typed<float, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, bias, relu, out, stream);
+    if (dtype == CGNN_F64)
+        return gather_typed<double, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, bias, relu, out, stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_reconstruct: dtype must be f32 or f64");
+}
+
+extern "C" int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int dtype,
+                                         const void *grad, const void *output,
+                                         const int32_t *offsets, const int32_t *perm,
+                                         const int32_t *sorted_id, int relu, void *reps_grad,
+                                         void *workspace, size_t workspace_bytes,
+                                         cgnn_stream_t stream) {
+    CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 0, "cgnn_reconstruct_backward: bad size");
+    CGNN_REQUIRE(dtype == CGNN_F32 || dtype == CGNN_F64, "cgnn_reconstruct_backward: dtype must be f32 or f64");
+    if (F == 0 || groups == 0) return CGNN_OK;
+    CGNN_REQUIRE(offsets && reps_grad, "cgnn_reconstruct_backward: null array");
+    CGNN_REQUIRE(N == 0 || (grad && perm && sorted_id), "cgnn_reconstruct_backward: null array");
+    CGNN_REQUIRE(!relu || N == 0 || output, "cgnn_reconstruct_backward: relu needs the saved output");
+    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id);
+    return spmm_members(&A, dtype, grad, output, reps_grad, F, relu != 0, workspace, workspace_bytes,
+                        stream);
+}
+
+extern "C" int cgnn_copy_bytes(const void *src, void *dst, size_t n, cgnn_stream_t stream) {
+    CGNN_REQUIRE(n % 16 == 0, "cgnn_copy_bytes: size must be a multiple of 16");
+    if (n == 0) return CGNN_OK;
+    CGNN_REQUIRE(src && dst, "cgnn_copy_bytes: null pointer");
+    size_t blocks = (n / 16 + kBlock - 1) / kBlock;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                       static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), n / 16);
+    return check_launch("copy_bytes");
+}

@@ -1,0 +1,639 @@
+// CSR SpMM for gfx950 (wave64): Y (+)= A * X with dense row-major X, Y of width F.
+//
+// Geometry shared by all kernels here.  A "lane group" of LPR consecutive lanes
+// (LPR a power of two, 4..64) owns one output row at a time; lane l of the group
+// holds VEC consecutive features starting at (tile*LPR + l)*VEC for TILES tiles, so a
+// group reads and writes LPR*VEC*sizeof(T) contiguous bytes per tile: 512 B per wave
+// instruction when VEC*sizeof(T) = 16 (global_load_dwordx4) and LPR*... covers a row.
+// Features beyond LPR*VEC*TILES are covered by blockIdx.y.  Index data are wave-uniform
+// when LPR == 64, so the compiler fetches them through the scalar unit.
+//
+// Two schedules:
+//   * row schedule  -- a lane group per row, entries summed in ascending order; the
+//     result is bit-identical to the sequential CPU sum of the reference
+//     (src/runtime/csrc/sparse/cpu/spmm_cpu.cpp:48-68): products and sums are rounded
+//     separately (this file is built with -ffp-contract=off).
+//   * nnz schedule  -- a lane group per run of seg_nnz consecutive non-zeros (rows of
+//     any length cost the same).  Rows that end inside the run are written by the run;
+//     the part of a row that continues into the next run is stored as a carry row and
+//     added by spmm_fixup_kernel, which walks the carries of one row in ascending run
+//     order.  No atomics anywhere, so results are reproducible run to run.
+//
+// X may alias Y when accumulating (rule levels are updated in place, reference
+// layer/CompressgnnSPMM.py:56-58), so X and Y carry no __restrict__; a row that is
+// written is never gathered in the same launch (levels only read earlier levels).
+#include "common.h"
+
+namespace cgnn {
+namespace {
+
+constexpr int kUnroll = 8;        // gathers in flight per lane and tile
+constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
+
+enum { MODE_VAL = 0, MODE_UNIT = 1, MODE_RELU_MASK = 2 };
+
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) Pack {
+    T v[VEC];
+};
+
+template <typename T>
+struct SpmmArgs {
+    const int32_t *__restrict__ rowptr;
+    const int32_t *__restrict__ colidx;
+    const int32_t *__restrict__ rowidx;
+    const T *__restrict__ val;
+    const T *X;   // gathered matrix (may alias Y)
+    const T *M;   // MODE_RELU_MASK: rows of X are zeroed where M <= 0
+    T *Y;
+    int32_t *carry_row;  // [nseg] row a run carries into, or -1
+    T *carry;            // [nseg x F]
+    int64_t F;
+    int32_t rows;
+    int32_t nnz;
+    int32_t nseg;
+    int32_t seg_nnz;
+    int32_t accumulate;
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> load_pack(const T *p) {
+    return *reinterpret_cast<const Pack<T, VEC> *>(p);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void store_pack(T *p, const Pack<T, VEC> &x) {
+    *reinterpret_cast<Pack<T, VEC> *>(p) = x;
+}
+
+// Per-lane feature offsets of the TILES tiles; foff[t] < 0 marks a tile beyond F.
+template <int VEC, int LPR, int TILES>
+__device__ __forceinline__ void feature_offsets(int64_t F, int lane, int64_t foff[TILES]) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        int64_t f = ((int64_t)(blockIdx.y * TILES + t) * LPR + lane) * VEC;
+        foff[t] = f < F ? f : -1;
+    }
+}
+
+template <typename T, int VEC, int TILES>
+__device__ __forceinline__ void zero_acc(Pack<T, VEC> acc[TILES]) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[t].v[i] = T(0);
+}
+
+// Y[row] = (accumulate ? Y[row] : 0) + acc
+template <typename T, int VEC, int TILES>
+__device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_t foff[TILES],
+                                          const Pack<T, VEC> acc[TILES], int accumulate) {
+    T *yrow = Y + (int64_t)row * F;
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        if (foff[t] < 0) continue;
+        Pack<T, VEC> o;
+        if (accumulate) {
+            o = load_pack<T, VEC>(yrow + foff[t]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) o.v[i] = T(0);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o.v[i] = o.v[i] + acc[t].v[i];
+        store_pack<T, VEC>(yrow + foff[t], o);
+    }
+}
+
+// Gather one feature tile of row c of X (masked by M in MODE_RELU_MASK).
+template <typename T, int VEC, int MODE>
+__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int64_t foff) {
+    Pack<T, VEC> x;
+    if (foff < 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = T(0);
+        return x;
+    }
+    const int64_t off = (int64_t)c * a.F + foff;
+    x = load_pack<T, VEC>(a.X + off);
+    if constexpr (MODE == MODE_RELU_MASK) {
+        Pack<T, VEC> m = load_pack<T, VEC>(a.M + off);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = (m.v[i] <= T(0)) ? T(0) : x.v[i];
+    }
+    return x;
+}
+
+template <typename T, int VEC, int TILES, int MODE>
+__device__ __forceinline__ void accumulate_entry(Pack<T, VEC> acc[TILES],
+                                                 const Pack<T, VEC> x[TILES], T w) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            if constexpr (MODE == MODE_VAL)
+                acc[t].v[i] = acc[t].v[i] + x[t].v[i] * w;
+            else
+                acc[t].v[i] = acc[t].v[i] + x[t].v[i];
+        }
+}
+
+// ---------------------------------------------------------------- row schedule --
+template <typename T, int VEC, int LPR, int TILES, int MODE>
+__global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
+    constexpr int GPB = kBlock / LPR;
+    const int lane = threadIdx.x % LPR;
+    int row = blockIdx.x * GPB + threadIdx.x / LPR;
+    if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
+    if (row >= a.rows) return;
+    int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
+    int64_t foff[TILES];
+    feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
+    Pack<T, VEC> acc[TILES];
+    zero_acc<T, VEC, TILES>(acc);
+    if (e0 == e1) {
+        if (!a.accumulate) write_row<T, VEC, TILES>(a.Y, a.F, row, foff, acc, 0);
+        return;
+    }
+    for (int e = e0; e < e1; e += kUnroll) {
+        int c[kUnroll];
+        T w[kUnroll];
+        Pack<T, VEC> x[kUnroll][TILES];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int idx = min(e + u, e1 - 1);
+            c[u] = a.colidx[idx];
+            w[u] = a.val ? a.val[idx] : T(1);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], foff[t]);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            if (e + u < e1) accumulate_entry<T, VEC, TILES, MODE>(acc, x[u], w[u]);
+    }
+    write_row<T, VEC, TILES>(a.Y, a.F, row, foff, acc, a.accumulate);
+}
+
+// Two blocks over the same rows in one pass: Y[row] = (sum A0 row) + (sum A1 row).
+template <typename T>
+struct PairArgs {
+    SpmmArgs<T> a0, a1;
+};
+
+template <typename T, int VEC, int LPR, int TILES>
+__device__ __forceinline__ void row_sum(const SpmmArgs<T> &a, int row, const int64_t foff[TILES],
+                                        Pack<T, VEC> acc[TILES]) {
+    int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
+    for (int e = e0; e < e1; e += kUnroll) {
+        int c[kUnroll];
+        T w[kUnroll];
+        Pack<T, VEC> x[kUnroll][TILES];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int idx = min(e + u, e1 - 1);
+            c[u] = a.colidx[idx];
+            w[u] = a.val ? a.val[idx] : T(1);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE_VAL>(a, c[u], foff[t]);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            if (e + u < e1) accumulate_entry<T, VEC, TILES, MODE_VAL>(acc, x[u], w[u]);
+    }
+}
+
+template <typename T, int VEC, int LPR, int TILES>
+__global__ __launch_bounds__(kBlock) void spmm_pair_kernel(PairArgs<T> p) {
+    constexpr int GPB = kBlock / LPR;
+    const int lane = threadIdx.x % LPR;
+    int row = blockIdx.x * GPB + threadIdx.x / LPR;
+    if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
+    if (row >= p.a0.rows) return;
+    int64_t foff[TILES];
+    feature_offsets<VEC, LPR, TILES>(p.a0.F, lane, foff);
+    Pack<T, VEC> s0[TILES], s1[TILES];
+    zero_acc<T, VEC, TILES>(s0);
+    zero_acc<T, VEC, TILES>(s1);
+    row_sum<T, VEC, LPR, TILES>(p.a0, row, foff, s0);
+    row_sum<T, VEC, LPR, TILES>(p.a1, row, foff, s1);
+    // (0 + s0) + s1, the order of two successive accumulating calls.
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) s0[t].v[i] = (T(0) + s0[t].v[i]) + s1[t].v[i];
+    write_row<T, VEC, TILES>(p.a0.Y, p.a0.F, row, foff, s0, 0);
+}
+
+// ---------------------------------------------------------------- nnz schedule --
+template <typename T, int VEC, int LPR, int TILES, int MODE>
+__global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
+    constexpr int GPB = kBlock / LPR;
+    const int lane = threadIdx.x % LPR;
+    int seg = blockIdx.x * GPB + threadIdx.x / LPR;
+    if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
+    if (seg >= a.nseg) return;
+    const int e0 = seg * a.seg_nnz;
+    const int e1 = min(e0 + a.seg_nnz, a.nnz);
+    int64_t foff[TILES];
+    feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
+    Pack<T, VEC> acc[TILES];
+    zero_acc<T, VEC, TILES>(acc);
+    int cur = a.rowidx[e0];
+    for (int e = e0; e < e1; e += kUnroll) {
+        int r[kUnroll], c[kUnroll];
+        T w[kUnroll];
+        Pack<T, VEC> x[kUnroll][TILES];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int idx = min(e + u, e1 - 1);
+            r[u] = a.rowidx[idx];
+            c[u] = a.colidx[idx];
+            if constexpr (MODE == MODE_VAL) w[u] = a.val[idx];
+            else w[u] = T(1);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], foff[t]);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (e + u < e1) {
+                if (r[u] != cur) {
+                    // row `cur` ends inside this run: finish it here
+                    write_row<T, VEC, TILES>(a.Y, a.F, cur, foff, acc, a.accumulate);
+                    zero_acc<T, VEC, TILES>(acc);
+                    cur = r[u];
+                }
+                accumulate_entry<T, VEC, TILES, MODE>(acc, x[u], w[u]);
+            }
+        }
+    }
+    const bool continues = (e1 < a.nnz) && (a.rowidx[e1] == cur);
+    if (continues) {
+        T *crow = a.carry + (int64_t)seg * a.F;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+            if (foff[t] >= 0) store_pack<T, VEC>(crow + foff[t], acc[t]);
+    } else {
+        write_row<T, VEC, TILES>(a.Y, a.F, cur, foff, acc, a.accumulate);
+    }
+    if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = continues ? cur : -1;
+}
+
+// Adds the carries of every row that straddles runs, in ascending run order, and
+// (when not accumulating) clears the rows that have no entries.  Work item i < nseg
+// handles run i if it is the first carry of its row; work item i < rows handles row i
+// if it is empty.  The two sets of rows are disjoint.
+template <typename T, int VEC, int LPR, int TILES>
+__global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
+    constexpr int GPB = kBlock / LPR;
+    const int lane = threadIdx.x % LPR;
+    int item = blockIdx.x * GPB + threadIdx.x / LPR;
+    if constexpr (LPR == kWave) item = __builtin_amdgcn_readfirstlane(item);
+    int64_t foff[TILES];
+    feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
+    Pack<T, VEC> acc[TILES];
+    if (item < a.nseg) {
+        const int r = a.carry_row[item];
+        if (r >= 0 && (item == 0 || a.carry_row[item - 1] != r)) {
+            zero_acc<T, VEC, TILES>(acc);
+            int s = item;
+            do {
+                const T *crow = a.carry + (int64_t)s * a.F;
+#pragma unroll
+                for (int t = 0; t < TILES; ++t)
+                    if (foff[t] >= 0) {
+                        Pack<T, VEC> cval = load_pack<T, VEC>(crow + foff[t]);
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) acc[t].v[i] = acc[t].v[i] + cval.v[i];
+                    }
+                ++s;
+            } while (s < a.nseg && a.carry_row[s] == r);
+            write_row<T, VEC, TILES>(a.Y, a.F, r, foff, acc, 1);
+        }
+    }
+    if (!a.accumulate && item < a.rows) {
+        if (a.rowptr[item] == a.rowptr[item + 1]) {
+            zero_acc<T, VEC, TILES>(acc);
+            write_row<T, VEC, TILES>(a.Y, a.F, item, foff, acc, 0);
+        }
+    }
+}
+
+// ------------------------------------------------------------------- dispatch --
+struct Shape {
+    int vec, lpr, tiles, grid_y;
+};
+
+// Lane layout for a feature width: the widest vector the width and the pointers'
+// alignment allow, then as many lanes as a row needs (power of two, 4..64).
+template <typename T>
+Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, const void *p3) {
+    auto aligned = [&](size_t bytes) {
+        auto ok = [&](const void *p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0; };
+        return ok(p0) && ok(p1) && ok(p2) && ok(p3);
+    };
+    Shape s;
+    s.vec = 1;
+    if (sizeof(T) == 4) {
+        if (F % 4 == 0 && aligned(16)) s.vec = 4;
+        else if (F % 2 == 0 && aligned(8)) s.vec = 2;
+    }
+    const int64_t slots = F / s.vec;
+    int lpr = pow2_ceil(slots);
+    if (lpr < 4) lpr = 4;
+    if (lpr > 64) lpr = 64;
+    if (s.vec != 4 || sizeof(T) != 4) {
+        // fewer instantiations off the main path: 4, 16 or 64 lanes per row
+        lpr = lpr <= 4 ? 4 : (lpr <= 16 ? 16 : 64);
+    }
+    s.lpr = lpr;
+    s.tiles = (lpr == 64 && slots > 64 && sizeof(T) == 4) ? 2 : 1;
+    s.grid_y = (int)ceil_div(slots, (int64_t)s.lpr * s.tiles);
+    return s;
+}
+
+enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2, KIND_PAIR = 3 };
+
+template <typename T, int VEC, int LPR, int TILES>
+int launch_shape(int kind, int mode, const SpmmArgs<T> &a, const SpmmArgs<T> *a1, int64_t items,
+                 int grid_y, hipStream_t stream) {
+    constexpr int GPB = kBlock / LPR;
+    dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
+    if (grid.x == 0) return CGNN_OK;
+    switch (kind) {
+        case KIND_ROW:
+            hipLaunchKernelGGL((spmm_row_kernel<T, VEC, LPR, TILES, MODE_VAL>), grid, block, 0, stream, a);
+            break;
+        case KIND_NNZ:
+            if (mode == MODE_VAL)
+                hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_VAL>), grid, block, 0, stream, a);
+            else if (mode == MODE_UNIT)
+                hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_UNIT>), grid, block, 0, stream, a);
+            else
+                hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_RELU_MASK>), grid, block, 0, stream, a);
+            break;
+        case KIND_FIXUP:
+            hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR, TILES>), grid, block, 0, stream, a);
+            break;
+        case KIND_PAIR: {
+            PairArgs<T> p{a, *a1};
+            hipLaunchKernelGGL((spmm_pair_kernel<T, VEC, LPR, TILES>), grid, block, 0, stream, p);
+            break;
+        }
+    }
+    return check_launch("spmm launch");
+}
+
+#define CGNN_SHAPE_CASE(V, L, TL)                   \
+    if (s.vec == V && s.lpr == L && s.tiles == TL)  \
+        return launch_shape<T, V, L, TL>(kind, mode, a, a1, items, s.grid_y, stream);
+
+template <typename T>
+int launch(int kind, int mode, const Shape &s, const SpmmArgs<T> &a, const SpmmArgs<T> *a1,
+           int64_t items, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4) {
+        CGNN_SHAPE_CASE(4, 4, 1)
+        CGNN_SHAPE_CASE(4, 8, 1)
+        CGNN_SHAPE_CASE(4, 16, 1)
+        CGNN_SHAPE_CASE(4, 32, 1)
+        CGNN_SHAPE_CASE(4, 64, 1)
+        CGNN_SHAPE_CASE(4, 64, 2)
+        CGNN_SHAPE_CASE(2, 4, 1)
+        CGNN_SHAPE_CASE(2, 16, 1)
+        CGNN_SHAPE_CASE(2, 64, 1)
+        CGNN_SHAPE_CASE(2, 64, 2)
+        CGNN_SHAPE_CASE(1, 4, 1)
+        CGNN_SHAPE_CASE(1, 16, 1)
+        CGNN_SHAPE_CASE(1, 64, 1)
+        CGNN_SHAPE_CASE(1, 64, 2)
+    } else {
+        CGNN_SHAPE_CASE(1, 4, 1)
+        CGNN_SHAPE_CASE(1, 16, 1)
+        CGNN_SHAPE_CASE(1, 64, 1)
+    }
+    return fail(CGNN_EUNSUPPORTED, "spmm: no kernel for this lane layout");
+}
+
+int resolve_kernel(const cgnn_csr *A, int kernel) {
+    if (kernel == CGNN_SPMM_ROW || kernel == CGNN_SPMM_NNZ) return kernel;
+    // AUTO: rows are "near regular" when the longest one is a small multiple of the
+    // mean; otherwise balance by non-zeros.  Needs rowidx for the nnz schedule.
+    if (A->rowidx == nullptr) return CGNN_SPMM_ROW;
+    if (A->max_row_nnz <= 0) return CGNN_SPMM_NNZ;
+    const double mean = A->rows > 0 ? (double)A->nnz / (double)A->rows : 0.0;
+    const double limit = 8.0 * (mean < 8.0 ? 8.0 : mean);
+    return (double)A->max_row_nnz <= limit ? CGNN_SPMM_ROW : CGNN_SPMM_NNZ;
+}
+
+int seg_len(const cgnn_csr *A) {
+    int s = A->seg_nnz > 0 ? A->seg_nnz : kDefaultSeg;
+    return (s + kUnroll - 1) / kUnroll * kUnroll;
+}
+
+int check_csr(const cgnn_csr *A, const char *name) {
+    if (A == nullptr) return fail(CGNN_EINVAL, "spmm: null csr");
+    const int64_t lim = (int64_t)INT32_MAX - 65536;  // room for run ends past the last entry
+    if (A->rows < 0 || A->cols < 0 || A->nnz < 0 || A->rows >= lim || A->nnz >= lim || A->cols >= lim) {
+        set_error("%s: rows/cols/nnz must be in [0, 2^31 - 65536)", name);
+        return CGNN_EINVAL;
+    }
+    if (A->rowptr == nullptr || (A->nnz > 0 && A->colidx == nullptr)) {
+        set_error("%s: rowptr/colidx must not be null", name);
+        return CGNN_EINVAL;
+    }
+    return CGNN_OK;
+}
+
+template <typename T>
+SpmmArgs<T> make_args(const cgnn_csr *A, const void *X, const void *M, void *Y, int64_t F,
+                      int accumulate) {
+    SpmmArgs<T> a{};
+    a.rowptr = A->rowptr;
+    a.colidx = A->colidx;
+    a.rowidx = A->rowidx;
+    a.val = static_cast<const T *>(A->val);
+    a.X = static_cast<const T *>(X);
+    a.M = static_cast<const T *>(M);
+    a.Y = static_cast<T *>(Y);
+    a.F = F;
+    a.rows = (int32_t)A->rows;
+    a.nnz = (int32_t)A->nnz;
+    a.accumulate = accumulate ? 1 : 0;
+    return a;
+}
+
+size_t carry_row_bytes(int64_t nseg) { return align_up((size_t)nseg * sizeof(int32_t), 256); }
+
+template <typename T>
+int spmm_typed(const cgnn_csr *A, const void *X, const void *M, void *Y, int64_t F, int accumulate,
+               int kernel, int mode, void *ws, size_t ws_bytes, hipStream_t stream) {
+    if (A->rows == 0 || F == 0) return CGNN_OK;
+    SpmmArgs<T> a = make_args<T>(A, X, M, Y, F, accumulate);
+    kernel = resolve_kernel(A, kernel);
+    if (mode == MODE_RELU_MASK) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
+    if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;
+    if (kernel == CGNN_SPMM_ROW) {
+        Shape s = pick_shape<T>(F, X, Y, nullptr, nullptr);
+        return launch<T>(KIND_ROW, mode, s, a, nullptr, A->rows, stream);
+    }
+    if (A->nnz > 0 && A->rowidx == nullptr) return fail(CGNN_EINVAL, "spmm: nnz schedule needs rowidx");
+    const int seg = seg_len(A);
+    const int64_t nseg = ceil_div(A->nnz, seg);
+    const size_t need = carry_row_bytes(nseg) + (size_t)nseg * F * sizeof(T);
+    if (nseg > 0 && (ws == nullptr || ws_bytes < need)) {
+        set_error("spmm: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+        return CGNN_EWORKSPACE;
+    }
+    a.nseg = (int32_t)nseg;
+    a.seg_nnz = seg;
+    a.carry_row = static_cast<int32_t *>(ws);
+    a.carry = reinterpret_cast<T *>(static_cast<char *>(ws) + carry_row_bytes(nseg));
+    Shape s = pick_shape<T>(F, X, Y, a.carry, M);
+    if (nseg > 0) {
+        int rc = launch<T>(KIND_NNZ, mode, s, a, nullptr, nseg, stream);
+        if (rc != CGNN_OK) return rc;
+    }
+    const int64_t items = accumulate ? nseg : (nseg > A->rows ? nseg : A->rows);
+    return launch<T>(KIND_FIXUP, mode, s, a, nullptr, items, stream);
+}
+
+}  // namespace
+
+// Entry used by the cluster reductions (unit values, optional ReLU mask).
+int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, void *Y, int64_t F,
+                 bool relu_mask, void *ws, size_t ws_bytes, hipStream_t stream) {
+    const int mode = relu_mask ? MODE_RELU_MASK : MODE_UNIT;
+    if (dtype == CGNN_F32)
+        return spmm_typed<float>(A, X, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
+    if (dtype == CGNN_F64)
+        return spmm_typed<double>(A, X, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
+    return fail(CGNN_EUNSUPPORTED, "spmm: dtype must be f32 or f64");
+}
+
+}  // namespace cgnn
+
+using namespace cgnn;
+
+extern "C" size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dtype, int kernel) {
+    if (A == nullptr || A->nnz <= 0 || F <= 0) return 0;
+    if (resolve_kernel(A, kernel) == CGNN_SPMM_ROW) return 0;
+    const int64_t nseg = ceil_div(A->nnz, seg_len(A));
+    const size_t elt = dtype == CGNN_F64 ? 8 : 4;
+    return carry_row_bytes(nseg) + (size_t)nseg * (size_t)F * elt;
+}
+
+extern "C" int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
+                         int accumulate, int kernel, void *workspace, size_t workspace_bytes,
+                         cgnn_stream_t stream) {
+    int rc = check_csr(A, "cgnn_spmm");
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(F >= 0, "cgnn_spmm: F must be non-negative");
+    if (A->rows == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(Y != nullptr, "cgnn_spmm: Y is null");
+    CGNN_REQUIRE(A->nnz == 0 || X != nullptr, "cgnn_spmm: X is null");
+    CGNN_REQUIRE(kernel >= CGNN_SPMM_AUTO && kernel <= CGNN_SPMM_NNZ, "cgnn_spmm: unknown kernel id");
+    if (dtype == CGNN_F32)
+        return spmm_typed<float>(A, X, nullptr, Y, F, accumulate, kernel, MODE_VAL, workspace,
+                                 workspace_bytes, stream);
+    if (dtype == CGNN_F64)
+        return spmm_typed<double>(A, X, nullptr, Y, F, accumulate, kernel, MODE_VAL, workspace,
+                                  workspace_bytes, stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_spmm: dtype must be f32 or f64");
+}
+
+template <typename T>
+static int spmm_pair_typed(const cgnn_csr *A0, const void *X0, const cgnn_csr *A1, const void *X1,
+                           void *Y, int64_t F, hipStream_t stream) {
+    SpmmArgs<T> a0 = make_args<T>(A0, X0, nullptr, Y, F, 0);
+    SpmmArgs<T> a1 = make_args<T>(A1, X1, nullptr, Y, F, 0);
+    Shape s = pick_shape<T>(F, X0, X1, Y, nullptr);
+    return launch<T>(KIND_PAIR, MODE_VAL, s, a0, &a1, A0->rows, stream);
+}
+
+extern "C" int cgnn_spmm_pair(const cgnn_csr *A0, const void *X0, const cgnn_csr *A1,
+                              const void *X1, int dtype, void *Y, int64_t F,
+                              cgnn_stream_t stream) {
+    int rc = check_csr(A0, "cgnn_spmm_pair(A0)");
+    if (rc != CGNN_OK) return rc;
+    rc = check_csr(A1, "cgnn_spmm_pair(A1)");
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(A0->rows == A1->rows, "cgnn_spmm_pair: blocks must have the same number of rows");
+    CGNN_REQUIRE(F >= 0, "cgnn_spmm_pair: F must be non-negative");
+    if (A0->rows == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(Y != nullptr, "cgnn_spmm_pair: Y is null");
+    CGNN_REQUIRE((A0->nnz == 0 || X0 != nullptr) && (A1->nnz == 0 || X1 != nullptr),
+                 "cgnn_spmm_pair: X is null");
+    if (dtype == CGNN_F32) return spmm_pair_typed<float>(A0, X0, A1, X1, Y, F, stream);
+    if (dtype == CGNN_F64) return spmm_pair_typed<double>(A0, X0, A1, X1, Y, F, stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_spmm_pair: dtype must be f32 or f64");
+}
+
+// ------------------------------------------------------- CSR preparation -------
+namespace cgnn {
+namespace {
+
+__global__ void narrow_i64_kernel(const int64_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x)
+        dst[i] = (int32_t)src[i];
+}
+
+// rowidx[e] = largest r with rowptr[r] <= e (rows without entries are skipped).
+template <typename P>
+__global__ void expand_rows_kernel(const P *__restrict__ rowptr, int64_t rows, int64_t nnz,
+                                   int32_t *__restrict__ rowidx) {
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz;
+         e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t lo = 0, hi = rows;  // invariant: rowptr[lo] <= e < rowptr[hi]
+        while (hi - lo > 1) {
+            int64_t mid = (lo + hi) >> 1;
+            if ((int64_t)rowptr[mid] <= e) lo = mid;
+            else hi = mid;
+        }
+        rowidx[e] = (int32_t)lo;
+    }
+}
+
+unsigned grid_for(int64_t n) {
+    int64_t b = ceil_div(n, kBlock);
+    return (unsigned)(b > 16384 ? 16384 : b);
+}
+
+}  // namespace
+}  // namespace cgnn
+
+extern "C" int cgnn_csr_prepare_i64(int64_t rows, int64_t nnz, const int64_t *rowptr64,
+                                    const int64_t *col64, int32_t *rowptr32, int32_t *col32,
+                                    int32_t *rowidx, cgnn_stream_t stream) {
+    const int64_t lim = (int64_t)INT32_MAX - 65536;
+    CGNN_REQUIRE(rows >= 0 && nnz >= 0 && rows < lim && nnz < lim, "cgnn_csr_prepare_i64: sizes must be in [0, 2^31 - 65536)");
+    CGNN_REQUIRE(rowptr64 != nullptr, "cgnn_csr_prepare_i64: rowptr is null");
+    if (rowptr32) {
+        hipLaunchKernelGGL(narrow_i64_kernel, dim3(grid_for(rows + 1)), dim3(kBlock), 0, stream, rowptr64,
+                           rowptr32, rows + 1);
+    }
+    if (col32 && nnz > 0) {
+        CGNN_REQUIRE(col64 != nullptr, "cgnn_csr_prepare_i64: col is null");
+        hipLaunchKernelGGL(narrow_i64_kernel, dim3(grid_for(nnz)), dim3(kBlock), 0, stream, col64, col32, nnz);
+    }
+    if (rowidx && nnz > 0) {
+        hipLaunchKernelGGL(expand_rows_kernel<int64_t>, dim3(grid_for(nnz)), dim3(kBlock), 0, stream,
+                           rowptr64, rows, nnz, rowidx);
+    }
+    return check_launch("csr_prepare");
+}
+
+extern "C" int cgnn_csr_expand_rows(int64_t rows, int64_t nnz, const int32_t *rowptr, int32_t *rowidx,
+                                    cgnn_stream_t stream) {
+    const int64_t lim = (int64_t)INT32_MAX - 65536;
+    CGNN_REQUIRE(rows >= 0 && nnz >= 0 && rows < lim && nnz < lim, "cgnn_csr_expand_rows: sizes must be in [0, 2^31 - 65536)");
+    if (nnz == 0) return CGNN_OK;
+    CGNN_REQUIRE(rowptr && rowidx, "cgnn_csr_expand_rows: null array");
+    hipLaunchKernelGGL(expand_rows_kernel<int32_t>, dim3(grid_for(nnz)), dim3(kBlock), 0, stream, rowptr,
+                       rows, nnz, rowidx);
+    return check_launch("csr_expand_rows");
+}

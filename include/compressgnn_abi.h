@@ -1,0 +1,178 @@
+/*
+ * compressgnn_abi.h -- C ABI of the MI355X (gfx950) device library libcgnn_hip.so.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream; none takes
+ * a framework type, none allocates device memory and none synchronises with the host
+ * unless its comment says so.  All launches go to the stream that is passed
+ * (NULL = the device's null stream) on the device that is current in the calling
+ * thread.  Return value: CGNN_OK (0) or a CGNN_E* code; cgnn_last_error() then holds
+ * a message for the calling thread.
+ *
+ * The comments name the interface of the reference implementation
+ * (ZhengChenCS/CompressGNN, paths relative to its root) that each entry replaces.
+ *
+ * Index arrays on the device are int32 (row counts and non-zero counts must be below
+ * 2^31); offsets into feature matrices are computed in 64 bits.  Feature matrices are
+ * dense row-major with row stride F.
+ */
+#ifndef COMPRESSGNN_ABI_H
+#define COMPRESSGNN_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t *cgnn_stream_t; /* == hipStream_t */
+
+enum cgnn_status {
+    CGNN_OK = 0,
+    CGNN_EINVAL = 1,       /* bad argument (shape, null pointer, range)          */
+    CGNN_EWORKSPACE = 2,   /* workspace missing or smaller than *_workspace_bytes */
+    CGNN_ELAUNCH = 3,      /* HIP reported an error at launch                     */
+    CGNN_EUNSUPPORTED = 4  /* dtype / size outside what the kernels cover         */
+};
+
+enum cgnn_dtype { CGNN_F32 = 0, CGNN_F64 = 1 };
+
+/* Which SpMM schedule to run.
+ *   ROW: one lane group per row, entries of a row summed in ascending order
+ *        (bit-identical to the sequential CPU sum of src/runtime/csrc/sparse/cpu/spmm_cpu.cpp:48-68).
+ *   NNZ: fixed-length runs of non-zeros per lane group, rows that straddle runs are
+ *        completed by an ordered fix-up pass (deterministic, no atomics).
+ *   AUTO: chosen from cgnn_csr.max_row_nnz and the mean row length.
+ * These replace the six CUDA methods of src/runtime/csrc/sparse/cuda/spmm_gpu.cu:27-99
+ * and the Python heuristic layer/CompressgnnSPMM.py:14-19. */
+enum cgnn_spmm_kernel { CGNN_SPMM_AUTO = 0, CGNN_SPMM_ROW = 1, CGNN_SPMM_NNZ = 2 };
+
+/* A CSR block resident on the device.  rowidx[e] is the row of non-zero e
+ * (non-decreasing); it is needed by the NNZ schedule only and may be NULL when the
+ * ROW schedule is requested.  val == NULL means every stored value is 1. */
+typedef struct cgnn_csr {
+    int64_t rows;
+    int64_t cols;
+    int64_t nnz;
+    const int32_t *rowptr; /* [rows+1] */
+    const int32_t *colidx; /* [nnz]    */
+    const int32_t *rowidx; /* [nnz] or NULL */
+    const void *val;       /* [nnz] of the call's dtype, or NULL */
+    int32_t max_row_nnz;   /* longest row, 0 if unknown (AUTO then picks NNZ) */
+    int32_t seg_nnz;       /* NNZ schedule: non-zeros per lane group, 0 = default */
+} cgnn_csr;
+
+const char *cgnn_last_error(void);
+const char *cgnn_version(void);
+
+/* ------------------------------------------------------------------ SpMM ---- */
+
+/* Bytes of scratch cgnn_spmm needs for this block, feature width and schedule
+ * (the carry-out rows of the NNZ schedule).  0 for the ROW schedule. */
+size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dtype, int kernel);
+
+/* Y[rows x F] (+)= A * X[cols x F].
+ * accumulate == 0: every row of Y is written (empty rows become 0);
+ * accumulate != 0: Y += A*X, rows without entries are left untouched, and Y may be
+ * the same buffer as X provided no row that is written is also read (the in-place
+ * rule-level update of layer/CompressgnnSPMM.py:56-58).
+ * Replaces spmm_func / spmm_cuda: src/runtime/csrc/sparse/spmm.cpp:11-22,
+ * src/runtime/csrc/sparse/cuda/spmm_gpu.cu:8-107. */
+int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
+              int accumulate, int kernel, void *workspace, size_t workspace_bytes,
+              cgnn_stream_t stream);
+
+/* Y[rows x F] = A0 * X0 + A1 * X1 in one pass over the rows (A0 and A1 have the same
+ * number of rows).  Each row is summed as (sum over A0's entries) + (sum over A1's
+ * entries), which is the value the two-call sequence
+ *   out = spmm(v2r, rule_out, None); out = spmm(v2v, x, out)
+ * of layer/CompressgnnSPMM.py:59-60 (and 84-85 in backward) produces, without
+ * reading Y back.  ROW schedule only (A0/A1 rowidx unused). */
+int cgnn_spmm_pair(const cgnn_csr *A0, const void *X0, const cgnn_csr *A1, const void *X1,
+                   int dtype, void *Y, int64_t F, cgnn_stream_t stream);
+
+/* Widen-free preparation of a CSR given as int64 tensors (the layout
+ * src/runtime/csrc/sparse/cuda/spmm_gpu.cu:38-46 reads): converts rowptr/col to
+ * int32 and writes the row of every non-zero.  Any of the outputs may be NULL. */
+int cgnn_csr_prepare_i64(int64_t rows, int64_t nnz, const int64_t *rowptr64,
+                         const int64_t *col64, int32_t *rowptr32, int32_t *col32,
+                         int32_t *rowidx, cgnn_stream_t stream);
+
+/* rowidx[e] = row of non-zero e, from an int32 rowptr. */
+int cgnn_csr_expand_rows(int64_t rows, int64_t nnz, const int32_t *rowptr,
+                         int32_t *rowidx, cgnn_stream_t stream);
+
+/* ------------------------------------------------- transformation compression -- */
+
+/* Scratch for cgnn_lsh_scan: bytes needed for 2^bits buckets. */
+size_t cgnn_lsh_scan_workspace_bytes(int bits);
+
+/* Step 1 of the assignment (src/runtime/csrc/cluster/cuda/cluster_kernel.cu:136-142,
+ * CPU twin src/runtime/csrc/cluster/cpu/cluster_cpu.cpp:41-56): for every row i of
+ * X[N x F], h_j = sum_k X[i,k]*W[k,j] accumulated with fused multiply-add in
+ * ascending k starting from 0, code = sum_j (h_j > 0) << (bits-1-j);
+ * raw_code[i] = code and bucket_count[code] += 1.  bucket_count (2^bits int32) is
+ * cleared by this call.  W is [F x bits] row-major. */
+int cgnn_lsh_hash(int64_t N, int64_t F, int bits, int dtype, const void *X, const void *W,
+                  int32_t *raw_code, int32_t *bucket_count, cgnn_stream_t stream);
+
+/* Step 2: prefix[b] = number of occupied buckets with index <= b (inclusive scan,
+ * cluster_kernel.cu:143-145).  prefix[2^bits - 1] is the number of active buckets;
+ * the caller reads it back (the one host synchronisation of cluster_kernel.cu:147). */
+int cgnn_lsh_scan(int bits, const int32_t *bucket_count, int32_t *prefix, void *workspace,
+                  size_t workspace_bytes, cgnn_stream_t stream);
+
+/* Step 3 (cluster_kernel.cu:51-59,149-150): ids[i] = prefix[raw_code[i]] (1-based,
+ * int64) and counts[prefix[b]] = bucket_count[b] for occupied b.  counts has
+ * active+1 entries and must be zero on entry (entry 0 stays 0). */
+int cgnn_lsh_finish(int64_t N, int bits, const int32_t *raw_code, const int32_t *bucket_count,
+                    const int32_t *prefix, int64_t *ids, int32_t *counts, cgnn_stream_t stream);
+
+/* Member lists of the clusters: a stable counting sort of the rows by id.
+ * offsets[g] = first position of group g in perm (offsets has groups+1 entries),
+ * perm[p] = row, sorted_id[p] = its id; rows of one group appear in ascending order.
+ * This is the CSR the segmented reductions below run on; it replaces the per-element
+ * float atomics of sum_features / reconstruct_grad (cluster_kernel.cu:60-69,98-108). */
+size_t cgnn_cluster_members_workspace_bytes(int64_t N, int64_t groups);
+int cgnn_cluster_members(int64_t N, int64_t groups, const int64_t *ids, int32_t *offsets,
+                         int32_t *perm, int32_t *sorted_id, void *workspace,
+                         size_t workspace_bytes, cgnn_stream_t stream);
+
+/* reps[g,:] = (sum over members i of group g, ascending i, of X[i,:]) / max(counts[g],1).
+ * Replaces cluster_mean_cuda (cluster_kernel.cu:158-170). */
+size_t cgnn_cluster_mean_workspace_bytes(int64_t N, int64_t F, int64_t groups, int dtype);
+int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype, const void *X,
+                      const int32_t *offsets, const int32_t *perm, const int32_t *sorted_id,
+                      const int32_t *counts, void *reps, void *workspace,
+                      size_t workspace_bytes, cgnn_stream_t stream);
+
+/* dx[i,:] = grad[ids[i],:] / max(counts[ids[i]],1).
+ * Replaces cluster_mean_backward_cuda (cluster_kernel.cu:171-181). */
+int cgnn_cluster_mean_backward(int64_t N, int64_t F, int64_t groups, int dtype, const void *grad,
+                               const int64_t *ids, const int32_t *counts, void *dx,
+                               cgnn_stream_t stream);
+
+/* out[i,:] = act(reps[ids[i],:] + bias), act(v) = (relu && v < 0) ? 0 : v; bias may be
+ * NULL.  Replaces cluster_reconstruct_cuda (cluster_kernel.cu:182-195). */
+int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
+                     const int64_t *ids, const void *bias, int relu, void *out,
+                     cgnn_stream_t stream);
+
+/* reps_grad[g,:] = sum over members i of g (ascending) of
+ * ((relu && output[i,:] <= 0) ? 0 : grad[i,:]).
+ * Replaces cluster_reconstruct_backward_cuda (cluster_kernel.cu:196-208). */
+int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int dtype, const void *grad,
+                              const void *output, const int32_t *offsets, const int32_t *perm,
+                              const int32_t *sorted_id, int relu, void *reps_grad,
+                              void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
+
+/* --------------------------------------------------------------- utilities ---- */
+
+/* A plain device-to-device copy kernel of n bytes (n % 16 == 0); the calibration
+ * kernel for scaling profiler byte counters. */
+int cgnn_copy_bytes(const void *src, void *dst, size_t n, cgnn_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COMPRESSGNN_ABI_H */

@@ -1,0 +1,116 @@
+"""Parity of the transformation-compression kernels (through the C ABI) against the
+CPU oracle, on the grid of the reference's own test (tests/test_transformation.py:21-39):
+dtype x width x (n, bits).  Ids, counts and the active-bucket count are bit-exact; means,
+gradients and reconstructions are within 1e-6 + 1e-5|b| (float32)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from compressgnn_amd import abi
+from util import assert_within
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {np.float32: dict(rtol=1e-5, atol=1e-6), np.float64: dict(rtol=1e-12, atol=1e-13)}
+
+
+def _t(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("width", [0, 1, 31, 33, 100, 128, 602])
+@pytest.mark.parametrize("n,bits", [(1, 0), (67, 8), (257, 16), (1000, 5), (5000, 12), (300, 20)])
+def test_assign_mean_reconstruct(dtype, width, n, bits):
+    rng = np.random.default_rng(1000 * bits + width + n)
+    x = rng.standard_normal((n, width)).astype(dtype)
+    w = rng.standard_normal((width, bits)).astype(dtype)
+    want_ids, want_counts, want_active = oracle.assign(x, w, bits)
+    ids, counts, active = abi.lsh_assign(_t(x), _t(w), bits)
+    torch.cuda.synchronize()
+    assert active == want_active
+    assert ids.dtype == torch.int64 and counts.dtype == torch.int32
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert np.array_equal(counts.cpu().numpy(), want_counts)
+    if width == 0:
+        return
+    groups = active + 1
+    members = abi.cluster_members(ids, groups)
+    offsets, perm, sorted_id = (m.cpu().numpy() for m in members)
+    order = np.argsort(want_ids, kind="stable")
+    assert np.array_equal(perm, order.astype(np.int32))
+    assert np.array_equal(sorted_id, want_ids[order].astype(np.int32))
+    assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(want_counts)]).astype(np.int32))
+    tol = TOL[dtype]
+    reps = abi.cluster_mean(_t(x), members, counts)
+    assert_within(reps.cpu().numpy(), oracle.cluster_mean(x, want_ids, want_counts), **tol)
+    grad = rng.standard_normal((groups, width)).astype(dtype)
+    dx = abi.cluster_mean_backward(_t(grad), ids, counts)
+    assert np.array_equal(dx.cpu().numpy(), oracle.cluster_mean_backward(grad, want_ids, want_counts))
+    bias = rng.standard_normal(width).astype(dtype)
+    for relu in (False, True):
+        for b in (None, bias):
+            out = abi.reconstruct(_t(grad), ids, None if b is None else _t(b), relu)
+            want = oracle.reconstruct(grad, want_ids, b, relu)
+            assert np.array_equal(out.cpu().numpy(), want)
+            go = rng.standard_normal((n, width)).astype(dtype)
+            rg = abi.reconstruct_backward(_t(go), out, members, groups, relu)
+            assert_within(rg.cpu().numpy(), oracle.reconstruct_backward(go, want_ids, want, groups, relu), **tol)
+
+
+@pytest.mark.parametrize("bits", [0, 8, 24])
+def test_all_collide(bits):
+    """Known answer of the reference's test: every row in one bucket -> count == [0, 513]."""
+    x = torch.ones(513, 33, device=DEV)
+    w = torch.ones(33, bits, device=DEV)
+    ids, counts, active = abi.lsh_assign(x, w, bits)
+    assert active == 1 and counts.tolist() == [0, 513]
+    assert ids.unique().tolist() == [1]
+
+
+def test_empty_input():
+    x = torch.zeros(0, 8, device=DEV)
+    w = torch.randn(8, 8, device=DEV)
+    ids, counts, active = abi.lsh_assign(x, w, 8)
+    assert ids.numel() == 0 and active == 0 and counts.tolist() == [0]
+
+
+def test_ids_match_exact_integer_projection():
+    """Independent of any summation order: integer-valued data make every projection
+    exact, so the ids must equal those of a float64 matmul (the torch restatement in
+    the reference's test, tests/test_transformation.py:16-20)."""
+    rng = np.random.default_rng(3)
+    x = rng.integers(-4, 5, size=(4000, 37)).astype(np.float32)
+    w = rng.integers(-3, 4, size=(37, 11)).astype(np.float32)
+    h = x.astype(np.float64) @ w.astype(np.float64)
+    code = np.zeros(len(x), np.int64)
+    for j in range(11):
+        code = (code << 1) + (h[:, j] > 0)
+    uniq, inv = np.unique(code, return_inverse=True)
+    ids, counts, active = abi.lsh_assign(_t(x), _t(w), 11)
+    assert active == len(uniq)
+    assert np.array_equal(ids.cpu().numpy(), inv + 1)
+    assert np.array_equal(counts.cpu().numpy(), np.bincount(inv + 1, minlength=len(uniq) + 1))
+
+
+def test_large_cluster_sums():
+    """A few hot clusters (tens of thousands of members): rows of the member CSR span
+    hundreds of runs."""
+    rng = np.random.default_rng(9)
+    n, F = 60000, 100
+    ids_np = rng.choice([1, 2, 3, 7], size=n, p=[0.6, 0.3, 0.09, 0.01]).astype(np.int64)
+    counts_np = np.bincount(ids_np, minlength=9).astype(np.int32)
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    ids, counts = _t(ids_np), _t(counts_np)
+    members = abi.cluster_members(ids, 9)
+    reps = abi.cluster_mean(_t(x), members, counts).cpu().numpy()
+    want64 = oracle.cluster_mean(x.astype(np.float64), ids_np, counts_np)
+    np.testing.assert_allclose(reps, want64, rtol=1e-5, atol=1e-6)
+    again = abi.cluster_mean(_t(x), members, counts).cpu().numpy()
+    assert np.array_equal(reps, again)
+    out = rng.standard_normal((n, F)).astype(np.float32)
+    go = rng.standard_normal((n, F)).astype(np.float32)
+    rg = abi.reconstruct_backward(_t(go), _t(out), members, 9, True).cpu().numpy()
+    want = oracle.reconstruct_backward(go.astype(np.float64), ids_np, out.astype(np.float64), 9, True)
+    np.testing.assert_allclose(rg, want, rtol=1e-4, atol=1e-3)

@@ -1,0 +1,168 @@
+"""Parity of the HIP SpMM (through the C ABI) against the CPU oracle on the same seeded
+inputs.  Row schedule: bit-exact (same summation order as the reference's sequential
+CPU sum).  Nnz schedule: rows that fit in one run are bit-exact too; rows that straddle
+runs are re-associated, so the bar is |a-b| <= 1e-6 + 1e-5|b| on sym-normalised-like
+weights."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from compressgnn_amd import abi
+from util import assert_within, random_csr
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _run(vlist, elist, value, x, kernel, out0=None, seg=0):
+    rows = len(vlist) - 1
+    A = abi.DeviceCsr.from_host(rows, x.shape[0], vlist, elist, value, DEV, seg_nnz=seg)
+    X = torch.from_numpy(x).to(DEV)
+    if out0 is None:
+        Y = abi.spmm(A, X, None, False, kernel)
+    else:
+        Y = torch.from_numpy(out0.copy()).to(DEV)
+        abi.spmm(A, X, Y, True, kernel)
+    torch.cuda.synchronize()
+    return Y.cpu().numpy()
+
+
+@pytest.mark.parametrize("F", [1, 3, 4, 16, 31, 33, 64, 100, 128, 130, 256, 512, 602])
+@pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
+def test_spmm_matches_oracle(F, kernel):
+    rng = np.random.default_rng(100 + F)
+    rows, cols = 777, 500
+    vlist, elist, value = random_csr(rng, rows, cols, 6.0)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    want = oracle.spmm(vlist, elist, value, x)
+    got = _run(vlist, elist, value, x, kernel)
+    if kernel == abi.SPMM_ROW:
+        assert np.array_equal(got, want)
+    else:
+        assert_within(got, want)
+    # accumulate onto an existing output
+    out0 = rng.standard_normal((rows, F)).astype(np.float32)
+    want2 = oracle.spmm(vlist, elist, value, x, out0.copy())
+    got2 = _run(vlist, elist, value, x, kernel, out0)
+    if kernel == abi.SPMM_ROW:
+        assert np.array_equal(got2, want2)
+    else:
+        assert_within(got2, want2)
+
+
+@pytest.mark.parametrize("seg", [8, 64, 256])
+@pytest.mark.parametrize("F", [16, 128, 200])
+def test_spmm_nnz_long_rows(F, seg):
+    """Power-law rows: many rows straddle runs, some span dozens of runs."""
+    rng = np.random.default_rng(7 * seg + F)
+    rows, cols = 600, 900
+    vlist, elist, value = random_csr(rng, rows, cols, 4.0, skew=True)
+    value = (value * 0.05).astype(np.float32)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    want = oracle.spmm(vlist, elist, value, x)
+    got = _run(vlist, elist, value, x, abi.SPMM_NNZ, seg=seg)
+    assert_within(got, want)
+    out0 = rng.standard_normal((rows, F)).astype(np.float32)
+    want2 = oracle.spmm(vlist, elist, value, x, out0.copy())
+    got2 = _run(vlist, elist, value, x, abi.SPMM_NNZ, out0, seg=seg)
+    assert_within(got2, want2)
+    # reproducible run to run (no atomics)
+    again = _run(vlist, elist, value, x, abi.SPMM_NNZ, seg=seg)
+    assert np.array_equal(got, again)
+
+
+@pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
+def test_spmm_edge_cases(kernel):
+    rng = np.random.default_rng(5)
+    F = 8
+    x = rng.standard_normal((10, F)).astype(np.float32)
+    # no entries at all: fresh output is zero, accumulate leaves the output alone
+    vlist = np.zeros(6, np.int64)
+    got = _run(vlist, np.zeros(0, np.int64), np.zeros(0, np.float32), x, kernel)
+    assert got.shape == (5, F) and not got.any()
+    out0 = rng.standard_normal((5, F)).astype(np.float32)
+    got = _run(vlist, np.zeros(0, np.int64), np.zeros(0, np.float32), x, kernel, out0)
+    assert np.array_equal(got, out0)
+    # leading and trailing empty rows, one dense row
+    vlist = np.array([0, 0, 0, 10, 10, 10], np.int64)
+    elist = np.arange(10, dtype=np.int64)
+    value = np.ones(10, np.float32)
+    want = oracle.spmm(vlist, elist, value, x)
+    assert_within(_run(vlist, elist, value, x, kernel), want)
+    # zero rows
+    A = abi.DeviceCsr.from_host(0, 10, np.zeros(1, np.int64), np.zeros(0, np.int64), np.zeros(0, np.float32), DEV)
+    Y = abi.spmm(A, torch.from_numpy(x).to(DEV), None, False, kernel)
+    assert Y.shape == (0, F)
+
+
+def test_spmm_in_place_levels():
+    """out aliases the gathered matrix: rows that are written are never gathered
+    (the in-place rule-level update of the reference's propagation)."""
+    rng = np.random.default_rng(11)
+    R, F = 400, 64
+    # rows 200.. gather rows 0..199 only; rows 0..199 are empty
+    deg = np.concatenate([np.zeros(200, np.int64), rng.integers(1, 9, size=200)])
+    vlist = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    elist = rng.integers(0, 200, size=int(vlist[-1])).astype(np.int64)
+    value = np.ones(int(vlist[-1]), np.float32)
+    z = rng.standard_normal((R, F)).astype(np.float32)
+    want = oracle.spmm(vlist, elist, value, z.copy(), None)
+    want = z + want  # accumulate onto itself
+    for kernel in (abi.SPMM_ROW, abi.SPMM_NNZ):
+        A = abi.DeviceCsr.from_host(R, R, vlist, elist, value, DEV)
+        Z = torch.from_numpy(z).to(DEV)
+        abi.spmm(A, Z, Z, True, kernel)
+        torch.cuda.synchronize()
+        if kernel == abi.SPMM_ROW:
+            assert np.array_equal(Z.cpu().numpy(), want)
+        else:
+            assert_within(Z.cpu().numpy(), want)
+
+
+def test_spmm_pair_equals_two_calls():
+    rng = np.random.default_rng(13)
+    V, R, F = 500, 120, 128
+    a0 = random_csr(rng, V, R, 2.0)
+    a1 = random_csr(rng, V, V, 7.0)
+    xr = rng.standard_normal((R, F)).astype(np.float32)
+    xv = rng.standard_normal((V, F)).astype(np.float32)
+    want = oracle.spmm(*a0, xr)
+    want = oracle.spmm(*a1, xv, want)
+    A0 = abi.DeviceCsr.from_host(V, R, *a0, DEV)
+    A1 = abi.DeviceCsr.from_host(V, V, *a1, DEV)
+    got = abi.spmm_pair(A0, torch.from_numpy(xr).to(DEV), A1, torch.from_numpy(xv).to(DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_spmm_f64():
+    rng = np.random.default_rng(17)
+    rows, cols, F = 300, 200, 10
+    vlist, elist, value = random_csr(rng, rows, cols, 5.0, skew=True)
+    x = rng.standard_normal((cols, F))
+    want = oracle.spmm(vlist, elist, value.astype(np.float64), x)
+    for kernel in (abi.SPMM_ROW, abi.SPMM_NNZ):
+        A = abi.DeviceCsr.from_host(rows, cols, vlist, elist, value.astype(np.float64), DEV)
+        Y = abi.spmm(A, torch.from_numpy(x).to(DEV), None, False, kernel)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(Y.cpu().numpy(), want, rtol=1e-12, atol=1e-12)
+
+
+def test_csr_prepare_i64():
+    import ctypes
+    rng = np.random.default_rng(19)
+    vlist, elist, _ = random_csr(rng, 1000, 300, 3.0, skew=True)
+    rows, nnz = 1000, len(elist)
+    rp = torch.from_numpy(vlist).to(DEV)
+    ci = torch.from_numpy(elist).to(DEV)
+    rp32 = torch.empty(rows + 1, dtype=torch.int32, device=DEV)
+    ci32 = torch.empty(nnz, dtype=torch.int32, device=DEV)
+    ri = torch.empty(nnz, dtype=torch.int32, device=DEV)
+    abi.check(abi.lib().cgnn_csr_prepare_i64(abi.i64(rows), abi.i64(nnz), abi.ptr(rp), abi.ptr(ci),
+                                             abi.ptr(rp32), abi.ptr(ci32), abi.ptr(ri), abi.stream_of(rp)))
+    torch.cuda.synchronize()
+    assert np.array_equal(rp32.cpu().numpy(), vlist.astype(np.int32))
+    assert np.array_equal(ci32.cpu().numpy(), elist.astype(np.int32))
+    want = np.repeat(np.arange(rows), np.diff(vlist)).astype(np.int32)
+    assert np.array_equal(ri.cpu().numpy(), want)
