@@ -62,7 +62,7 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_kernel(LshArgs<T> a) {
         const int ks = min(a.slab, a.F - k0);  // multiple of VEC
         const int ks_v = ks / VEC;
         // magic division is exact for the full slab; a shorter last slab divides directly
-        const bool full = ks == a.slab;
+        const bool full = ks == a.slab && a.magic != 0;
         const int total = rows_here * ks_v;
         __syncthreads();
         for (int i = lane; i < total; i += kLshRows) {
@@ -159,7 +159,7 @@ int lsh_hash_typed(int64_t N, int64_t F, int bits, const void *X, const void *W,
     a.slab = slab;
     const int slab_v = slab / vec;
     a.stride_v = slab_v | 1;
-    a.magic = (uint32_t)((1ull << 32) / (uint32_t)slab_v) + 1u;
+    a.magic = slab_v > 1 ? (uint32_t)((1ull << 32) / (uint32_t)slab_v) + 1u : 0u;  // 0: divide directly
     if (wide) return dispatch_lsh<T, WIDE>(a, stream);
     return dispatch_lsh<T, 1>(a, stream);
 }

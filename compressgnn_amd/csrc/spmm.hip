@@ -13,11 +13,12 @@
 //     result is bit-identical to the sequential CPU sum of the reference
 //     (src/runtime/csrc/sparse/cpu/spmm_cpu.cpp:48-68): products and sums are rounded
 //     separately (this file is built with -ffp-contract=off).
-//   * nnz schedule  -- a lane group per run of seg_nnz consecutive non-zeros (rows of
-//     any length cost the same).  Rows that end inside the run are written by the run;
-//     the part of a row that continues into the next run is stored as a carry row and
-//     added by spmm_fixup_kernel, which walks the carries of one row in ascending run
-//     order.  No atomics anywhere, so results are reproducible run to run.
+//   * nnz schedule  -- a lane group per run of about seg_nnz consecutive non-zeros (rows
+//     of any length cost the same).  Rows of at most seg_nnz entries always lie inside
+//     one run and are summed exactly as in the row schedule.  Longer rows are cut at
+//     multiples of seg_nnz: the part that continues into the next run is stored as a
+//     carry row and added by spmm_fixup_kernel, which walks the carries of one row in
+//     ascending run order.  No atomics anywhere, so results are reproducible run to run.
 //
 // X may alias Y when accumulating (rule levels are updated in place, reference
 // layer/CompressgnnSPMM.py:56-58), so X and Y carry no __restrict__; a row that is
@@ -228,6 +229,18 @@ __global__ __launch_bounds__(kBlock) void spmm_pair_kernel(PairArgs<T> p) {
 }
 
 // ---------------------------------------------------------------- nnz schedule --
+// Run s covers the non-zeros [run_boundary(s*K), run_boundary((s+1)*K)).  A boundary
+// that falls inside a row of at most K entries is moved back to the start of that row,
+// so such rows are never split (and are summed in the same order as the row schedule);
+// only rows longer than K are cut, at multiples of K.  Runs hold fewer than 2K entries.
+template <typename T>
+__device__ __forceinline__ int run_boundary(const SpmmArgs<T> &a, int e) {
+    if (e >= a.nnz) return a.nnz;
+    const int r = a.rowidx[e];
+    const int s0 = a.rowptr[r];
+    return (a.rowptr[r + 1] - s0 <= a.seg_nnz) ? s0 : e;
+}
+
 template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
@@ -235,8 +248,12 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     int seg = blockIdx.x * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
     if (seg >= a.nseg) return;
-    const int e0 = seg * a.seg_nnz;
-    const int e1 = min(e0 + a.seg_nnz, a.nnz);
+    const int e0 = run_boundary(a, seg * a.seg_nnz);
+    const int e1 = run_boundary(a, (seg + 1) * a.seg_nnz);
+    if (e0 >= e1) {  // cannot happen for a well-formed CSR; keeps the fix-up pass consistent
+        if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = -1;
+        return;
+    }
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
     Pack<T, VEC> acc[TILES];

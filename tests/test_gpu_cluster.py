@@ -1,7 +1,10 @@
 """Parity of the transformation-compression kernels (through the C ABI) against the
 CPU oracle, on the grid of the reference's own test (tests/test_transformation.py:21-39):
-dtype x width x (n, bits).  Ids, counts and the active-bucket count are bit-exact; means,
-gradients and reconstructions are within 1e-6 + 1e-5|b| (float32)."""
+dtype x width x (n, bits).  Ids, counts, the active-bucket count, mean gradients and
+reconstructions are bit-exact.  Cluster sums (means, reconstruct gradients) are
+bit-exact for clusters of at most 64 members (one run of the segmented reduction) and
+within the reference test's own tolerance (atol 1e-5, rtol 1e-4 for float32,
+tests/test_transformation.py:14) for larger ones, whose sums are re-associated."""
 import numpy as np
 import pytest
 import torch
@@ -12,7 +15,7 @@ from util import assert_within
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-TOL = {np.float32: dict(rtol=1e-5, atol=1e-6), np.float64: dict(rtol=1e-12, atol=1e-13)}
+TOL = {np.float32: dict(rtol=1e-4, atol=1e-5), np.float64: dict(rtol=1e-12, atol=1e-13)}
 
 
 def _t(a):
@@ -43,8 +46,11 @@ def test_assign_mean_reconstruct(dtype, width, n, bits):
     assert np.array_equal(sorted_id, want_ids[order].astype(np.int32))
     assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(want_counts)]).astype(np.int32))
     tol = TOL[dtype]
-    reps = abi.cluster_mean(_t(x), members, counts)
-    assert_within(reps.cpu().numpy(), oracle.cluster_mean(x, want_ids, want_counts), **tol)
+    small = want_counts <= 64
+    reps = abi.cluster_mean(_t(x), members, counts).cpu().numpy()
+    want_reps = oracle.cluster_mean(x, want_ids, want_counts)
+    assert_within(reps, want_reps, **tol)
+    assert np.array_equal(reps[small], want_reps[small])
     grad = rng.standard_normal((groups, width)).astype(dtype)
     dx = abi.cluster_mean_backward(_t(grad), ids, counts)
     assert np.array_equal(dx.cpu().numpy(), oracle.cluster_mean_backward(grad, want_ids, want_counts))
@@ -55,8 +61,10 @@ def test_assign_mean_reconstruct(dtype, width, n, bits):
             want = oracle.reconstruct(grad, want_ids, b, relu)
             assert np.array_equal(out.cpu().numpy(), want)
             go = rng.standard_normal((n, width)).astype(dtype)
-            rg = abi.reconstruct_backward(_t(go), out, members, groups, relu)
-            assert_within(rg.cpu().numpy(), oracle.reconstruct_backward(go, want_ids, want, groups, relu), **tol)
+            rg = abi.reconstruct_backward(_t(go), out, members, groups, relu).cpu().numpy()
+            want_rg = oracle.reconstruct_backward(go, want_ids, want, groups, relu)
+            assert_within(rg, want_rg, **tol)
+            assert np.array_equal(rg[small], want_rg[small])
 
 
 @pytest.mark.parametrize("bits", [0, 8, 24])
