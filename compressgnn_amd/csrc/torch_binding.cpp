@@ -1,0 +1,501 @@
+// `compressgnn_runtime`: the Python-visible operator module, with the operator names,
+// argument order and error behaviour of the reference's extension
+// (ZhengChenCS/CompressGNN src/runtime/csrc/function.cpp:9-21).  Host code only: every
+// computation is a call into libcgnn_hip.so through the C ABI
+// (include/compressgnn_abi.h); torch supplies tensors, the caching allocator and the
+// current stream.  There is no CPU implementation behind these operators: CPU tensors
+// are rejected with an error.
+#include <ATen/hip/HIPContext.h>
+#include <c10/hip/HIPGuard.h>
+#include <torch/extension.h>
+
+#include <map>
+#include <memory>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "compressgnn_abi.h"
+
+namespace {
+
+using torch::Tensor;
+
+void ok(int rc, const char *what) {
+    TORCH_CHECK(rc == CGNN_OK, what, ": ", cgnn_last_error());
+}
+
+cgnn_stream_t current_stream(const Tensor &t) {
+    return reinterpret_cast<cgnn_stream_t>(at::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+int dtype_code(const Tensor &t) {
+    TORCH_CHECK(t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kFloat64,
+                "Only float32 and float64 are supported");
+    return t.scalar_type() == torch::kFloat32 ? CGNN_F32 : CGNN_F64;
+}
+
+void require_gpu(const Tensor &t, const char *name) {
+    TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor: this build of compressgnn_runtime has no CPU operators");
+}
+
+// ----------------------------------------------------------------- CSR blocks ----
+
+// A CSR block resident on the device in the layout the kernels read (int32 indices,
+// row of every non-zero), with its scratch buffers.  Built once per graph block.
+struct DeviceCsr {
+    int64_t rows = 0, cols = 0, nnz = 0;
+    Tensor rowptr, colidx, rowidx, val;
+    int32_t max_row_nnz = 0;
+    int32_t seg_nnz = 0;
+    std::map<std::tuple<int64_t, int, int>, Tensor> scratch;
+
+    cgnn_csr view() const {
+        cgnn_csr a{};
+        a.rows = rows;
+        a.cols = cols;
+        a.nnz = nnz;
+        a.rowptr = rowptr.data_ptr<int32_t>();
+        a.colidx = nnz ? colidx.data_ptr<int32_t>() : nullptr;
+        a.rowidx = (nnz && rowidx.defined()) ? rowidx.data_ptr<int32_t>() : nullptr;
+        a.val = (nnz && val.defined()) ? val.data_ptr() : nullptr;
+        a.max_row_nnz = max_row_nnz;
+        a.seg_nnz = seg_nnz;
+        return a;
+    }
+
+    Tensor workspace(int64_t F, int dtype, int kernel, size_t *bytes) {
+        cgnn_csr a = view();
+        *bytes = cgnn_spmm_workspace_bytes(&a, F, dtype, kernel);
+        auto key = std::make_tuple(F, dtype, kernel);
+        auto it = scratch.find(key);
+        if (it == scratch.end() || (size_t)it->second.numel() < *bytes) {
+            Tensor t = torch::empty({(int64_t)std::max<size_t>(*bytes, 1)},
+                                    rowptr.options().dtype(torch::kUInt8));
+            scratch[key] = t;
+            return t;
+        }
+        return it->second;
+    }
+};
+
+// rowptr/col: int64 or int32 tensors on any device; value: float tensor or undefined.
+std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows,
+                                    int64_t cols, torch::Device device, int64_t seg_nnz) {
+    TORCH_CHECK(device.is_cuda(), "DeviceCsr lives on a GPU");
+    TORCH_CHECK(rowptr.dim() == 1 && col.dim() == 1 && rowptr.numel() == rows + 1, "rowptr must have rows+1 entries");
+    auto blk = std::make_shared<DeviceCsr>();
+    blk->rows = rows;
+    blk->cols = cols;
+    blk->nnz = col.numel();
+    blk->seg_nnz = (int32_t)seg_nnz;
+    const int64_t lim = (int64_t)INT32_MAX - 65536;
+    TORCH_CHECK(rows < lim && cols < lim && blk->nnz < lim, "block exceeds the int32 index range of the kernels");
+    c10::hip::HIPGuard guard(device);
+    Tensor rp = rowptr.to(device).contiguous();
+    Tensor ci = col.to(device).contiguous();
+    auto i32 = torch::TensorOptions().device(device).dtype(torch::kInt32);
+    if (rp.scalar_type() == torch::kInt64) {
+        blk->rowptr = torch::empty({rows + 1}, i32);
+        blk->colidx = torch::empty({blk->nnz}, i32);
+        blk->rowidx = torch::empty({blk->nnz}, i32);
+        TORCH_CHECK(ci.scalar_type() == torch::kInt64, "rowptr and col must have the same integer type");
+        ok(cgnn_csr_prepare_i64(rows, blk->nnz, rp.data_ptr<int64_t>(), blk->nnz ? ci.data_ptr<int64_t>() : nullptr,
+                                blk->rowptr.data_ptr<int32_t>(), blk->nnz ? blk->colidx.data_ptr<int32_t>() : nullptr,
+                                blk->nnz ? blk->rowidx.data_ptr<int32_t>() : nullptr, current_stream(rp)),
+           "csr_prepare");
+    } else {
+        TORCH_CHECK(rp.scalar_type() == torch::kInt32 && ci.scalar_type() == torch::kInt32,
+                    "rowptr/col must be int64 or int32");
+        blk->rowptr = rp;
+        blk->colidx = ci;
+        blk->rowidx = torch::empty({blk->nnz}, i32);
+        ok(cgnn_csr_expand_rows(rows, blk->nnz, rp.data_ptr<int32_t>(),
+                                blk->nnz ? blk->rowidx.data_ptr<int32_t>() : nullptr, current_stream(rp)),
+           "csr_expand_rows");
+    }
+    if (value.has_value() && value->defined()) {
+        TORCH_CHECK(value->numel() == blk->nnz, "value must have one entry per non-zero");
+        blk->val = value->to(device).contiguous();
+    }
+    if (rows > 0) {
+        Tensor lens = blk->rowptr.slice(0, 1, rows + 1) - blk->rowptr.slice(0, 0, rows);
+        blk->max_row_nnz = lens.max().item<int32_t>();  // one host read per block, at build time
+    }
+    return blk;
+}
+
+int kernel_of_method(const std::string &method) {
+    // The reference's six GPU method strings (src/runtime/csrc/sparse/cuda/spmm_gpu.cu:27-31)
+    // and its two CPU ones are accepted; "rowbalance*" asks for the row schedule,
+    // "nnzbalance*" for the nnz schedule, "auto" lets the block's row lengths decide.
+    if (method == "auto") return CGNN_SPMM_AUTO;
+    if (method == "rowbalance" || method == "rowbalance_parreduce" || method == "rowbalance_seqreduce" ||
+        method == "rowbalance_rowcache")
+        return CGNN_SPMM_ROW;
+    if (method == "nnzbalance" || method == "nnzbalance_parreduce" || method == "nnzbalance_seqreduce" ||
+        method == "nnzbalance_rowcache")
+        return CGNN_SPMM_NNZ;
+    TORCH_CHECK(false, "Invalid SpMM method: ", method);
+}
+
+// out (+)= A * mat.  `out` undefined: a fresh [rows, F] tensor is returned.
+Tensor block_spmm(DeviceCsr &A, const Tensor &mat, c10::optional<Tensor> optional_out, int kernel) {
+    require_gpu(mat, "mat");
+    TORCH_CHECK(mat.is_contiguous(), "mat must be contiguous");
+    TORCH_CHECK(mat.dim() == 2, "mat must be a matrix");
+    TORCH_CHECK(mat.size(0) == A.cols, "mat has ", mat.size(0), " rows, the block has ", A.cols, " columns");
+    TORCH_CHECK(!A.val.defined() || A.val.scalar_type() == mat.scalar_type(), "value and mat must have the same dtype");
+    c10::hip::HIPGuard guard(mat.device());
+    const int64_t F = mat.size(1);
+    const int dtype = dtype_code(mat);
+    Tensor out;
+    int accumulate = 0;
+    if (optional_out.has_value() && optional_out->defined()) {
+        // like the reference (spmm_gpu.cu:20-22) a non-contiguous out is copied, so the
+        // caller must use the returned tensor
+        out = optional_out->contiguous();
+        require_gpu(out, "out");
+        TORCH_CHECK(out.dim() == 2 && out.size(0) == A.rows && out.size(1) == F && out.scalar_type() == mat.scalar_type(),
+                    "out must be [rows, F] of mat's dtype");
+        accumulate = 1;
+    } else {
+        out = torch::empty({A.rows, F}, mat.options());
+    }
+    if (A.rows == 0 || F == 0) return out;
+    size_t bytes = 0;
+    Tensor ws = A.workspace(F, dtype, kernel, &bytes);
+    cgnn_csr a = A.view();
+    ok(cgnn_spmm(&a, dtype, mat.data_ptr(), out.data_ptr(), F, accumulate, kernel, ws.data_ptr(), bytes,
+                 current_stream(mat)),
+       "spmm");
+    return out;
+}
+
+// spmm_func of the reference (src/runtime/csrc/sparse/spmm.cpp:11-22): CSR given as
+// int64 tensors, prepared on every call.  Graph blocks that are used repeatedly should
+// be wrapped in a DeviceCsr once instead.
+Tensor spmm_func(Tensor vlist, Tensor elist, Tensor value, Tensor mat, std::string method,
+                 c10::optional<Tensor> optional_out) {
+    require_gpu(mat, "mat");
+    require_gpu(vlist, "vlist");
+    require_gpu(elist, "elist");
+    require_gpu(value, "value");
+    const int kernel = kernel_of_method(method);
+    TORCH_CHECK(vlist.scalar_type() == torch::kInt64 && elist.scalar_type() == torch::kInt64,
+                "vlist and elist must be int64");
+    auto blk = make_csr(vlist, elist, value, vlist.size(-1) - 1, mat.size(0), mat.device(), 0);
+    return block_spmm(*blk, mat, optional_out, kernel);
+}
+
+// ------------------------------------------------------- compressed propagation ----
+
+// The device form of a CompressGraph (loader/compress_graph.py:6-43 of the reference):
+// the three vertex/rule blocks, the rule levels and their transposes.
+struct PropagationPlan {
+    std::shared_ptr<DeviceCsr> v2v, v2r, r2v, v2v_t, v2r_t, r2v_t;
+    std::vector<std::shared_ptr<DeviceCsr>> r2r, r2r_t;
+    int64_t V = 0, R = 0;
+    bool fuse_final = true;  // last two stages in one pass (cgnn_spmm_pair)
+    int kernel = CGNN_SPMM_AUTO;
+};
+
+Tensor final_stage(PropagationPlan &p, DeviceCsr &from_rules, const Tensor &rule_x, DeviceCsr &from_vertices,
+                   const Tensor &x) {
+    const int64_t F = x.size(1);
+    if (p.fuse_final) {
+        Tensor out = torch::empty({from_vertices.rows, F}, x.options());
+        if (out.numel() == 0) return out;
+        cgnn_csr a0 = from_rules.view(), a1 = from_vertices.view();
+        ok(cgnn_spmm_pair(&a0, rule_x.data_ptr(), &a1, x.data_ptr(), dtype_code(x), out.data_ptr(), F,
+                          current_stream(x)),
+           "spmm_pair");
+        return out;
+    }
+    Tensor out = block_spmm(from_rules, rule_x, c10::nullopt, p.kernel);
+    return block_spmm(from_vertices, x, out, p.kernel);
+}
+
+// layer/CompressgnnSPMM.py:43-62 of the reference.
+Tensor propagate_forward(PropagationPlan &p, Tensor x) {
+    require_gpu(x, "x");
+    TORCH_CHECK(x.dim() == 2 && x.size(0) == p.V, "x must be [vertex_cnt, F]");
+    x = x.contiguous();
+    c10::hip::HIPGuard guard(x.device());
+    Tensor rule_out = block_spmm(*p.r2v, x, c10::nullopt, p.kernel);
+    for (auto &level : p.r2r) rule_out = block_spmm(*level, rule_out, rule_out, p.kernel);
+    return final_stage(p, *p.v2r, rule_out, *p.v2v, x);
+}
+
+// layer/CompressgnnSPMM.py:65-86 (the working branch, lines 80-85).
+Tensor propagate_backward(PropagationPlan &p, Tensor grad) {
+    require_gpu(grad, "grad");
+    TORCH_CHECK(grad.dim() == 2 && grad.size(0) == p.V, "grad must be [vertex_cnt, F]");
+    grad = grad.contiguous();
+    c10::hip::HIPGuard guard(grad.device());
+    Tensor rule_g = block_spmm(*p.v2r_t, grad, c10::nullopt, p.kernel);
+    for (auto it = p.r2r_t.rbegin(); it != p.r2r_t.rend(); ++it) rule_g = block_spmm(**it, rule_g, rule_g, p.kernel);
+    return final_stage(p, *p.r2v_t, rule_g, *p.v2v_t, grad);
+}
+
+// ---------------------------------------------------- transformation compression ----
+
+int bucket_size(int64_t bits) {
+    TORCH_CHECK(bits >= 0 && bits <= 30, "Hash bits must be in [0,30]");
+    return 1 << bits;
+}
+
+void check_float(const Tensor &x) {
+    TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.is_contiguous(), "Expected contiguous GPU matrix");
+    TORCH_CHECK(x.scalar_type() == torch::kFloat32 || x.scalar_type() == torch::kFloat64,
+                "Only float32 and float64 are supported");
+}
+void check_index(const Tensor &index, torch::Device device) {
+    TORCH_CHECK(index.device() == device && index.dim() == 1 && index.is_contiguous() &&
+                    index.scalar_type() == torch::kInt64,
+                "Expected contiguous int64 index on input device");
+}
+void check_count(const Tensor &count, torch::Device device) {
+    TORCH_CHECK(count.device() == device && count.dim() == 1 && count.is_contiguous() &&
+                    count.scalar_type() == torch::kInt32 && count.numel() >= 1,
+                "Expected nonempty int32 counts on input device");
+}
+
+// cluster_workspace_cuda (src/runtime/csrc/cluster/cuda/cluster_kernel.cu:111-117):
+// [bucket counts int32[2^bits], prefix int32[2^bits], scan scratch uint8[...]].
+std::vector<Tensor> cluster_workspace(Tensor input, int64_t bits) {
+    check_float(input);
+    c10::hip::HIPGuard guard(input.device());
+    const int n = bucket_size(bits);
+    auto ints = input.options().dtype(torch::kInt32);
+    return {torch::empty({n}, ints), torch::empty({n}, ints),
+            torch::empty({(int64_t)cgnn_lsh_scan_workspace_bytes((int)bits)}, input.options().dtype(torch::kUInt8))};
+}
+
+// cluster_assign_cuda (cluster_kernel.cu:118-153).
+std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, int64_t bits,
+                                                   std::vector<Tensor> workspace) {
+    check_float(input);
+    check_float(planes);
+    c10::hip::HIPGuard guard(input.device());
+    const int n = bucket_size(bits);
+    TORCH_CHECK(planes.device() == input.device() && planes.scalar_type() == input.scalar_type() &&
+                    planes.size(0) == input.size(1) && planes.size(1) == bits,
+                "Hash plane shape/device/dtype mismatch");
+    TORCH_CHECK(input.size(0) <= INT_MAX, "Node count exceeds int32 bucket count capacity");
+    TORCH_CHECK(workspace.size() == 3, "Expected bucket, prefix and scan workspaces");
+    for (int i = 0; i < 3; ++i)
+        TORCH_CHECK(workspace[i].device() == input.device() && workspace[i].dim() == 1 && workspace[i].is_contiguous(),
+                    "Workspace device/shape mismatch");
+    const size_t scan_bytes = cgnn_lsh_scan_workspace_bytes((int)bits);
+    TORCH_CHECK(workspace[0].scalar_type() == torch::kInt32 && workspace[1].scalar_type() == torch::kInt32 &&
+                    workspace[0].numel() == n && workspace[1].numel() == n &&
+                    workspace[2].scalar_type() == torch::kUInt8 && (size_t)workspace[2].numel() >= scan_bytes,
+                "Workspace dtype/capacity mismatch");
+    const int64_t N = input.size(0);
+    Tensor ids = torch::empty({N}, input.options().dtype(torch::kInt64));
+    if (N == 0) return {ids, torch::zeros({1}, workspace[0].options()), 0};
+    auto stream = current_stream(input);
+    Tensor raw = torch::empty({N}, workspace[0].options());
+    Tensor buckets = workspace[0], prefix = workspace[1];
+    ok(cgnn_lsh_hash(N, input.size(1), (int)bits, dtype_code(input), input.data_ptr(), planes.data_ptr(),
+                     raw.data_ptr<int32_t>(), buckets.data_ptr<int32_t>(), stream),
+       "lsh_hash");
+    ok(cgnn_lsh_scan((int)bits, buckets.data_ptr<int32_t>(), prefix.data_ptr<int32_t>(), workspace[2].data_ptr(),
+                     (size_t)workspace[2].numel(), stream),
+       "lsh_scan");
+    // One scalar read, only when assignments are refreshed (cluster_kernel.cu:146-147).
+    const int active = prefix.select(0, n - 1).item<int>();
+    Tensor counts = torch::zeros({active + 1}, buckets.options());
+    ok(cgnn_lsh_finish(N, (int)bits, raw.data_ptr<int32_t>(), buckets.data_ptr<int32_t>(), prefix.data_ptr<int32_t>(),
+                       ids.data_ptr<int64_t>(), counts.data_ptr<int32_t>(), stream),
+       "lsh_finish");
+    return {ids, counts, (int64_t)active};
+}
+
+// cluster_forward (src/runtime/csrc/cluster/cluster.cpp:12-30): int32 ids and the
+// number of active buckets.
+std::tuple<Tensor, int64_t> cluster_forward(Tensor input, Tensor random_vectors, int64_t param_h) {
+    TORCH_CHECK(input.dim() == 2 && random_vectors.dim() == 2 && input.is_contiguous() && random_vectors.is_contiguous(),
+                "Expected contiguous matrices");
+    TORCH_CHECK(param_h >= 0 && param_h <= 30 && random_vectors.size(0) == input.size(1) && random_vectors.size(1) == param_h,
+                "Invalid hash plane shape/bits");
+    TORCH_CHECK(input.device() == random_vectors.device() && input.scalar_type() == random_vectors.scalar_type(),
+                "Hash device/dtype mismatch");
+    TORCH_CHECK(input.scalar_type() == torch::kFloat32 || input.scalar_type() == torch::kFloat64,
+                "Expected float32/float64 features");
+    require_gpu(input, "input");
+    auto result = cluster_assign(input, random_vectors, param_h, cluster_workspace(input, param_h));
+    return {std::get<0>(result).to(torch::kInt32), std::get<2>(result)};
+}
+
+// Member lists of `groups` clusters: [offsets int32[groups+1], perm int32[N], sorted_id int32[N]].
+std::vector<Tensor> cluster_members(Tensor index, int64_t groups) {
+    TORCH_CHECK(index.is_cuda(), "index must be a GPU tensor");
+    check_index(index, index.device());
+    TORCH_CHECK(groups >= 1, "groups must be positive");
+    c10::hip::HIPGuard guard(index.device());
+    const int64_t N = index.numel();
+    auto i32 = index.options().dtype(torch::kInt32);
+    Tensor offsets = torch::empty({groups + 1}, i32), perm = torch::empty({N}, i32), sorted = torch::empty({N}, i32);
+    const size_t bytes = cgnn_cluster_members_workspace_bytes(N, groups);
+    Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, index.options().dtype(torch::kUInt8));
+    ok(cgnn_cluster_members(N, groups, N ? index.data_ptr<int64_t>() : nullptr, offsets.data_ptr<int32_t>(),
+                            N ? perm.data_ptr<int32_t>() : nullptr, N ? sorted.data_ptr<int32_t>() : nullptr,
+                            ws.data_ptr(), bytes, current_stream(index)),
+       "cluster_members");
+    return {offsets, perm, sorted};
+}
+
+std::vector<Tensor> members_or_build(const c10::optional<std::vector<Tensor>> &members, const Tensor &index,
+                                     int64_t groups) {
+    if (members.has_value() && !members->empty()) {
+        const auto &m = *members;
+        TORCH_CHECK(m.size() == 3 && m[0].numel() == groups + 1 && m[1].numel() == index.numel() &&
+                        m[2].numel() == index.numel() && m[0].scalar_type() == torch::kInt32 &&
+                        m[1].scalar_type() == torch::kInt32 && m[2].scalar_type() == torch::kInt32 &&
+                        m[0].device() == index.device(),
+                    "member lists do not match index/groups");
+        return m;
+    }
+    return cluster_members(index, groups);
+}
+
+// cluster_mean_cuda (cluster_kernel.cu:158-170).  `members` (from cluster_members, for
+// the same index) avoids rebuilding the member lists on every call.
+Tensor cluster_mean(Tensor input, Tensor index, Tensor count, c10::optional<std::vector<Tensor>> members) {
+    check_float(input);
+    check_index(index, input.device());
+    check_count(count, input.device());
+    TORCH_CHECK(index.numel() == input.size(0), "Input/index length mismatch");
+    c10::hip::HIPGuard guard(input.device());
+    const int64_t N = input.size(0), F = input.size(1), groups = count.numel();
+    if (input.numel() == 0) return torch::zeros({groups, F}, input.options());
+    auto m = members_or_build(members, index, groups);
+    Tensor out = torch::empty({groups, F}, input.options());
+    const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(input));
+    Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, input.options().dtype(torch::kUInt8));
+    ok(cgnn_cluster_mean(N, F, groups, dtype_code(input), input.data_ptr(), m[0].data_ptr<int32_t>(),
+                         m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(), count.data_ptr<int32_t>(), out.data_ptr(),
+                         ws.data_ptr(), bytes, current_stream(input)),
+       "cluster_mean");
+    return out;
+}
+
+// cluster_mean_backward_cuda (cluster_kernel.cu:171-181).
+Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count) {
+    check_float(grad);
+    check_index(index, grad.device());
+    check_count(count, grad.device());
+    TORCH_CHECK(grad.size(0) == count.numel(), "Gradient/count shape mismatch");
+    c10::hip::HIPGuard guard(grad.device());
+    Tensor out = torch::empty({index.numel(), grad.size(1)}, grad.options());
+    if (out.numel() == 0) return out;
+    ok(cgnn_cluster_mean_backward(index.numel(), grad.size(1), count.numel(), dtype_code(grad), grad.data_ptr(),
+                                  index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), out.data_ptr(),
+                                  current_stream(grad)),
+       "cluster_mean_backward");
+    return out;
+}
+
+// cluster_reconstruct_cuda (cluster_kernel.cu:182-195).
+Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias, bool relu) {
+    check_float(reps);
+    check_index(index, reps.device());
+    if (bias.has_value())
+        TORCH_CHECK(bias->device() == reps.device() && bias->scalar_type() == reps.scalar_type() && bias->dim() == 1 &&
+                        bias->numel() == reps.size(1) && bias->is_contiguous(),
+                    "Invalid reconstruction bias");
+    c10::hip::HIPGuard guard(reps.device());
+    Tensor out = torch::empty({index.numel(), reps.size(1)}, reps.options());
+    if (out.numel() == 0) return out;
+    ok(cgnn_reconstruct(index.numel(), reps.size(1), reps.size(0), dtype_code(reps), reps.data_ptr(),
+                        index.data_ptr<int64_t>(), bias.has_value() ? bias->data_ptr() : nullptr, relu ? 1 : 0,
+                        out.data_ptr(), current_stream(reps)),
+       "cluster_reconstruct");
+    return out;
+}
+
+// cluster_reconstruct_backward_cuda (cluster_kernel.cu:196-208).
+Tensor cluster_reconstruct_backward(Tensor grad, Tensor index, Tensor output, int64_t groups, bool relu,
+                                    c10::optional<std::vector<Tensor>> members) {
+    check_float(grad);
+    check_index(index, grad.device());
+    check_float(output);
+    TORCH_CHECK(groups >= 0 && output.sizes() == grad.sizes() && output.device() == grad.device() &&
+                    output.scalar_type() == grad.scalar_type() && index.numel() == grad.size(0),
+                "Invalid reconstruction gradient");
+    c10::hip::HIPGuard guard(grad.device());
+    const int64_t N = grad.size(0), F = grad.size(1);
+    if (grad.numel() == 0 || groups == 0) return torch::zeros({groups, F}, grad.options());
+    auto m = members_or_build(members, index, groups);
+    Tensor out = torch::empty({groups, F}, grad.options());
+    const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(grad));
+    Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, grad.options().dtype(torch::kUInt8));
+    ok(cgnn_reconstruct_backward(N, F, groups, dtype_code(grad), grad.data_ptr(), output.data_ptr(),
+                                 m[0].data_ptr<int32_t>(), m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(),
+                                 relu ? 1 : 0, out.data_ptr(), ws.data_ptr(), bytes, current_stream(grad)),
+       "cluster_reconstruct_backward");
+    return out;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    namespace py = pybind11;
+    m.doc() = "CompressGNN runtime operators for MI355X (HIP kernels behind a C ABI)";
+    // the reference's operator set (src/runtime/csrc/function.cpp:10-20)
+    m.def("spmm_func", &spmm_func, "spmm function", py::arg("vlist"), py::arg("elist"), py::arg("value"),
+          py::arg("mat"), py::arg("method"), py::arg("optional_out") = py::none());
+    m.def("cluster_forward", &cluster_forward, "CompressGNN cluster forward");
+    m.def("cluster_workspace", &cluster_workspace);
+    m.def("cluster_assign", &cluster_assign);
+    m.def("cluster_mean", &cluster_mean, py::arg("input"), py::arg("index"), py::arg("count"),
+          py::arg("members") = py::none());
+    m.def("cluster_mean_backward", &cluster_mean_backward);
+    m.def("cluster_reconstruct", &cluster_reconstruct);
+    m.def("cluster_reconstruct_backward", &cluster_reconstruct_backward, py::arg("grad"), py::arg("index"),
+          py::arg("output"), py::arg("groups"), py::arg("relu"), py::arg("members") = py::none());
+    // additions of this build
+    m.def("cluster_members", &cluster_members, "member lists (offsets, perm, sorted_id) of the clusters");
+    m.def("version", []() { return std::string(cgnn_version()); });
+    py::class_<DeviceCsr, std::shared_ptr<DeviceCsr>>(m, "DeviceCsr")
+        .def(py::init([](Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows, int64_t cols,
+                         torch::Device device, int64_t seg_nnz) {
+                 return make_csr(rowptr, col, value, rows, cols, device, seg_nnz);
+             }),
+             py::arg("rowptr"), py::arg("col"), py::arg("value"), py::arg("rows"), py::arg("cols"),
+             py::arg("device"), py::arg("seg_nnz") = 0)
+        .def_readonly("rows", &DeviceCsr::rows)
+        .def_readonly("cols", &DeviceCsr::cols)
+        .def_readonly("nnz", &DeviceCsr::nnz)
+        .def_readonly("max_row_nnz", &DeviceCsr::max_row_nnz)
+        .def_readwrite("seg_nnz", &DeviceCsr::seg_nnz)
+        .def_readonly("rowptr", &DeviceCsr::rowptr)
+        .def_readonly("colidx", &DeviceCsr::colidx)
+        .def_readonly("rowidx", &DeviceCsr::rowidx)
+        .def_readonly("val", &DeviceCsr::val)
+        .def("spmm",
+             [](DeviceCsr &self, Tensor mat, c10::optional<Tensor> out, std::string method) {
+                 return block_spmm(self, mat, out, kernel_of_method(method));
+             },
+             py::arg("mat"), py::arg("out") = py::none(), py::arg("method") = "auto");
+    py::class_<PropagationPlan, std::shared_ptr<PropagationPlan>>(m, "PropagationPlan")
+        .def(py::init([](std::shared_ptr<DeviceCsr> v2v, std::shared_ptr<DeviceCsr> v2r, std::shared_ptr<DeviceCsr> r2v,
+                         std::vector<std::shared_ptr<DeviceCsr>> r2r, std::shared_ptr<DeviceCsr> v2v_t,
+                         std::shared_ptr<DeviceCsr> v2r_t, std::shared_ptr<DeviceCsr> r2v_t,
+                         std::vector<std::shared_ptr<DeviceCsr>> r2r_t) {
+                 auto p = std::make_shared<PropagationPlan>();
+                 p->v2v = v2v; p->v2r = v2r; p->r2v = r2v; p->r2r = r2r;
+                 p->v2v_t = v2v_t; p->v2r_t = v2r_t; p->r2v_t = r2v_t; p->r2r_t = r2r_t;
+                 p->V = v2v->rows; p->R = r2v->rows;
+                 TORCH_CHECK(r2r.size() == r2r_t.size(), "levels and transposed levels differ in number");
+                 return p;
+             }))
+        .def_readwrite("fuse_final", &PropagationPlan::fuse_final)
+        .def_property("method",
+                      [](PropagationPlan &p) { return p.kernel == CGNN_SPMM_ROW ? "rowbalance" : p.kernel == CGNN_SPMM_NNZ ? "nnzbalance" : "auto"; },
+                      [](PropagationPlan &p, std::string mth) { p.kernel = kernel_of_method(mth); })
+        .def("forward", &propagate_forward)
+        .def("backward", &propagate_backward);
+}

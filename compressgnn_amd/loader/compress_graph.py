@@ -1,0 +1,78 @@
+"""CompressGraph: the on-device format of a compressed graph -- three CSR blocks
+(vertex->vertex, vertex->rule, rule->vertex), the rule->rule levels, and expanded
+degrees.  Same fields, constructor and to() as the reference's
+loader/compress_graph.py:6-57; on a GPU it additionally carries the propagation plan
+(int32 index arrays, rows of non-zeros, transposes) that the HIP kernels read."""
+import _paths  # noqa: F401
+import torch
+
+from compressgnn_offline import gen_degree, hybird_partition, topo_partition
+from sparse_csr import SparseCSR
+
+
+class CompressGraph():
+    def __init__(self, vlist, elist, value, vertex_cnt):
+        """vlist/elist/value: CSC of the (vertex_cnt + rule_cnt)-square compressed matrix,
+        i.e. row i lists the parents of node i, vertex parents first."""
+        as_np = lambda t: t.detach().cpu().numpy() if torch.is_tensor(t) else t
+        v2v, v2r, r2v, r2r = hybird_partition(as_np(vlist), as_np(elist), as_np(value), vertex_cnt)
+        r2r_list = topo_partition(r2r[0], r2r[1], r2r[2])
+        rule_cnt = len(r2v[0]) - 1
+        t = torch.from_numpy
+        self.vertex_cnt, self.rule_cnt = int(vertex_cnt), int(rule_cnt)
+        self.v2v_graph = SparseCSR(t(v2v[0]), t(v2v[1]), t(v2v[2]), (vertex_cnt, vertex_cnt))
+        self.v2r_graph = SparseCSR(t(v2r[0]), t(v2r[1]), t(v2r[2]), (vertex_cnt, rule_cnt))
+        self.r2v_graph = SparseCSR(t(r2v[0]), t(r2v[1]), t(r2v[2]), (rule_cnt, vertex_cnt))
+        self.step = len(r2r_list)
+        self.r2r_graph = [SparseCSR(t(lv[0]), t(lv[1]), t(lv[2]), (rule_cnt, rule_cnt)) for lv in r2r_list]
+        vertex_degree, rule_degree = gen_degree(v2v[0], v2v[1], v2r[0], v2r[1], r2v[0], r2v[1],
+                                                [lv[0] for lv in r2r_list], [lv[1] for lv in r2r_list])
+        self.vertex_degree = t(vertex_degree)
+        self.rule_degree = t(rule_degree)
+        self._plan = None
+
+    def __repr__(self):
+        return 'CompressGraph'
+
+    def blocks(self):
+        return [self.v2v_graph, self.v2r_graph, self.r2v_graph] + list(self.r2r_graph)
+
+    def to(self, device):
+        device = torch.device(device)
+        if device.type == "cuda":
+            for g in self.blocks():
+                g.csc()  # transposes are built on the host, before the blocks move
+        self.v2v_graph = self.v2v_graph.to(device)
+        self.v2r_graph = self.v2r_graph.to(device)
+        self.r2v_graph = self.r2v_graph.to(device)
+        for s in range(self.step):
+            self.r2r_graph[s] = self.r2r_graph[s].to(device)
+        self.vertex_degree = self.vertex_degree.to(device)
+        self.rule_degree = self.rule_degree.to(device)
+        self._plan = None
+        return self
+
+    @property
+    def device(self):
+        return self.v2v_graph.device
+
+    def plan(self):
+        """The device-side propagation plan (built on first use after to(device))."""
+        if self._plan is None:
+            import compressgnn_runtime as rt
+            dev = self.device
+            if dev.type != "cuda":
+                raise RuntimeError("CompressGraph.plan(): move the graph to a GPU first (graph.to('cuda'))")
+
+            def fwd(g):
+                rp, ci, val = g.csr()
+                return rt.DeviceCsr(rp, ci, val, g.sparse_size(0), g.sparse_size(1), dev)
+
+            def bwd(g):
+                cp, row, val = g.csc()
+                return rt.DeviceCsr(cp, row, val, g.sparse_size(1), g.sparse_size(0), dev)
+
+            self._plan = rt.PropagationPlan(
+                fwd(self.v2v_graph), fwd(self.v2r_graph), fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
+                bwd(self.v2v_graph), bwd(self.v2r_graph), bwd(self.r2v_graph), [bwd(g) for g in self.r2r_graph])
+        return self._plan

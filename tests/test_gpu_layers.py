@@ -1,0 +1,233 @@
+"""End-to-end parity of the drop-in layers on the GPU: CompressgnnData -> CompressGraph ->
+KPropagate forward/backward against (a) the CPU oracle's 4-stage chain on the same blocks
+and (b) the plain, uncompressed A^T x of the same graph; Compressgnn_Cluster /
+Compressgnn_Reconstruct forward/backward against the oracle and torch autograd of the
+index_select composition (the checks of the reference's tests/test_transformation.py)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path[:0] = [os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compressgnn_amd", "layer"),
+                os.path.join(ROOT, "compressgnn_amd", "loader")]
+
+import oracle
+from util import assert_within
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _np_blocks(graph):
+    def csr(g):
+        rp, ci, val = g.csr()
+        return rp.cpu().numpy(), ci.cpu().numpy(), val.cpu().numpy()
+
+    def csc(g):
+        cp, row, val = g.csc()
+        return cp.cpu().numpy(), row.cpu().numpy(), val.cpu().numpy()
+
+    fwd = dict(v2v=csr(graph.v2v_graph), v2r=csr(graph.v2r_graph), r2v=csr(graph.r2v_graph),
+               r2r=[csr(g) for g in graph.r2r_graph])
+    bwd = dict(v2v_t=csc(graph.v2v_graph), v2r_t=csc(graph.v2r_graph), r2v_t=csc(graph.r2v_graph),
+               r2r_t=[csc(g) for g in graph.r2r_graph])
+    return fwd, bwd
+
+
+def _make_data(kind, F, normalize=True, freq=16, seed=0):
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    rng = np.random.default_rng(seed)
+    if kind == "chung_lu":
+        v, e = off.gen_chung_lu(2708, 10500, 2.5, seed)
+    elif kind == "copy":
+        v, e = off.gen_copy_model(6000, 9.8, 0.7, seed)
+    elif kind == "blocks":
+        n = 64
+        v = np.arange(n + 1, dtype=np.int64) * 32
+        e = np.tile(np.arange(32, dtype=np.int64), n)
+    V = len(v) - 1
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    mask = np.ones(V, dtype=bool)
+    data = CompressgnnData(x, (v, e), np.zeros(V, np.int64), mask, mask, mask, add_self_loop=True,
+                           normalize=normalize, graph_type="csr", min_pair_frequency=freq)
+    return data, (v, e)
+
+
+def _plain_transpose_product(v, e, x, normalize):
+    """out = A_hat^T x of the uncompressed graph with self loops and (optionally)
+    symmetric normalisation, in float64."""
+    import compressgnn_offline as off
+    v2, e2 = off.add_self_loop_csr(v, e)
+    V = len(v2) - 1
+    src = np.repeat(np.arange(V), np.diff(v2))
+    if normalize:
+        d = off.get_norm_degree(e2, V).astype(np.float64)
+        w = d[src] * d[e2]
+    else:
+        w = np.ones(len(e2))
+    out = np.zeros((V, x.shape[1]))
+    np.add.at(out, e2, w[:, None] * x[src].astype(np.float64))
+    return out
+
+
+@pytest.mark.parametrize("kind,freq", [("chung_lu", 16), ("chung_lu", 3), ("copy", 3), ("blocks", 16)])
+@pytest.mark.parametrize("normalize", [True, False])
+@pytest.mark.parametrize("F", [128, 16])
+def test_propagate_forward_backward(kind, freq, normalize, F):
+    from KPropagate import KPropagate
+    data, (v, e) = _make_data(kind, F, normalize, freq)
+    graph = data.edge_index
+    fwd_blocks, bwd_blocks = _np_blocks(graph)
+    x_np = data.x.numpy().copy()
+    if kind != "chung_lu" or freq == 3:
+        assert data.rule_cnt > 0
+    want = oracle.compress_spmm_forward(fwd_blocks, x_np) if data.rule_cnt else oracle.spmm(*fwd_blocks["v2v"], x_np)
+    plain = _plain_transpose_product(v, e, x_np, normalize)
+    # the oracle's compressed chain equals the uncompressed product (re-association only)
+    np.testing.assert_allclose(want, plain, rtol=2e-4, atol=2e-5 if normalize else 2e-3)
+
+    data.to(DEV)
+    prop = KPropagate()
+    x = data.x.detach().clone().requires_grad_()
+    out = prop(x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    g_np = np.random.default_rng(5).standard_normal(out.shape).astype(np.float32)
+    (gx,) = torch.autograd.grad(out, x, torch.from_numpy(g_np).to(DEV))
+    torch.cuda.synchronize()
+    want_gx = (oracle.compress_spmm_backward(bwd_blocks, g_np) if data.rule_cnt
+               else oracle.spmm(*bwd_blocks["v2v_t"], g_np))
+    tol = dict(rtol=1e-5, atol=1e-6) if normalize else dict(rtol=1e-5, atol=1e-4)
+    assert_within(out.detach().cpu().numpy(), want, **tol)
+    assert_within(gx.cpu().numpy(), want_gx, **tol)
+    # adjoint identity <A x, g> == <x, A^T g> in float64 on the GPU results
+    lhs = float((out.detach().cpu().numpy().astype(np.float64) * g_np).sum())
+    rhs = float((x_np.astype(np.float64) * gx.cpu().numpy()).sum())
+    assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs))
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+@pytest.mark.parametrize("method", ["rowbalance", "nnzbalance", "auto"])
+def test_propagate_schedules_agree(fuse, method):
+    from CompressgnnSPMM import compress_spmm
+    data, _ = _make_data("copy", 64, True, 3)
+    fwd_blocks, _ = _np_blocks(data.edge_index)
+    want = oracle.compress_spmm_forward(fwd_blocks, data.x.numpy())
+    data.to(DEV)
+    plan = data.edge_index.plan()
+    plan.fuse_final, plan.method = fuse, method
+    out = compress_spmm(data.edge_index, data.x)
+    torch.cuda.synchronize()
+    assert_within(out.cpu().numpy(), want)
+    if method == "rowbalance":
+        assert np.array_equal(out.cpu().numpy(), want)  # sequential sums in every stage
+
+
+def test_spmm_func_int64_api():
+    """The reference's raw operator on int64 CSR tensors, all accepted method strings."""
+    import compressgnn_runtime as rt
+    from util import random_csr
+    rng = np.random.default_rng(2)
+    vlist, elist, value = random_csr(rng, 300, 200, 5.0, skew=True)
+    x = rng.standard_normal((200, 48)).astype(np.float32)
+    want = oracle.spmm(vlist, elist, value, x)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    for method in ["rowbalance_rowcache", "nnzbalance_rowcache", "rowbalance_parreduce", "nnzbalance_seqreduce"]:
+        out = rt.spmm_func(t(vlist), t(elist), t(value), t(x), method, None)
+        assert_within(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+        acc = t(np.ones((300, 48), np.float32))
+        ret = rt.spmm_func(t(vlist), t(elist), t(value), t(x), method, acc)
+        assert ret.data_ptr() == acc.data_ptr()
+        assert_within(acc.cpu().numpy(), want + 1, rtol=1e-5, atol=1e-5)
+    with pytest.raises(RuntimeError):
+        rt.spmm_func(t(vlist), t(elist), t(value), t(x), "no_such_method", None)
+    with pytest.raises(RuntimeError):
+        rt.spmm_func(torch.from_numpy(vlist), torch.from_numpy(elist), torch.from_numpy(value),
+                     torch.from_numpy(x), "rowbalance", None)
+
+
+def test_cluster_reconstruct_layers():
+    from CompressgnnCluster import Compressgnn_Cluster, Compressgnn_Cluster_Function, _Mean
+    from CompressgnnReconstruct import Compressgnn_Reconstruct
+    torch.manual_seed(26)
+    reconstruct = Compressgnn_Reconstruct()
+    idx = torch.tensor([1, 1, 3, 1, 3, 3], device=DEV)
+    count = torch.bincount(idx, minlength=5).int()
+    x = torch.randn(6, 5, device=DEV, dtype=torch.double, requires_grad=True)
+    assert torch.autograd.gradcheck(lambda a: _Mean.apply(a, idx, count), (x,), eps=1e-6, atol=1e-5, rtol=1e-3)
+    for dtype in [torch.float32, torch.float64]:
+        for width in [1, 31, 33, 128, 602]:
+            for relu in [None, 'relu']:
+                reps = torch.randn(5, width, device=DEV, dtype=dtype, requires_grad=True)
+                bias = torch.randn(width, device=DEV, dtype=dtype, requires_grad=True)
+                out = reconstruct(reps, idx, bias=bias, activation=relu)
+                ref = reps.index_select(0, idx) + bias
+                if relu:
+                    ref = ref.relu()
+                torch.testing.assert_close(out, ref, atol=1e-5, rtol=1e-4)
+                go = torch.randn_like(out)
+                a = torch.autograd.grad(out, (reps, bias), go)
+                b = torch.autograd.grad(ref, (reps, bias), go)
+                torch.testing.assert_close(a[0], b[0], atol=1e-5, rtol=1e-4)
+                torch.testing.assert_close(a[1], b[1], atol=1e-5, rtol=1e-4)
+    reps = torch.randn(5, 3, device=DEV, dtype=torch.double, requires_grad=True)
+    bias = torch.full((3,), 2., device=DEV, dtype=torch.double, requires_grad=True)
+    assert torch.autograd.gradcheck(lambda a, b: reconstruct(a, idx, b, 'relu'), (reps, bias), eps=1e-6,
+                                    atol=1e-5, rtol=1e-3)
+
+    def scatter_mean(x, index, groups):
+        s = torch.zeros(groups, x.size(1), device=x.device, dtype=x.dtype).index_add_(0, index, x)
+        c = torch.bincount(index, minlength=groups).clamp_min(1).to(x.dtype)
+        return s / c[:, None]
+
+    c = Compressgnn_Cluster(7, 4, device=DEV, refresh_interval=5)
+    ptr = None
+    for epoch in range(12):
+        x = torch.randn(19, 7, device=DEV, requires_grad=True)
+        out, index = c(x, epoch=epoch, cache_key='graph-A')
+        assert c.last_refreshed == (epoch % 5 == 0)
+        if epoch % 5:
+            assert index.data_ptr() == ptr
+        ptr = index.data_ptr()
+        ref = scatter_mean(x, index, out.size(0))
+        torch.testing.assert_close(out, ref, atol=1e-5, rtol=1e-4)
+        torch.testing.assert_close(torch.autograd.grad(out.square().sum(), x)[0],
+                                   torch.autograd.grad(ref.square().sum(), x)[0], atol=1e-5, rtol=1e-4)
+    assert c.refresh_count == 3
+    # two shared transforms, one reconstruction, all parameter gradients
+    layers = torch.nn.Sequential(torch.nn.Linear(7, 9), torch.nn.ReLU(), torch.nn.Linear(9, 3)).to(DEV)
+    x = torch.randn(19, 7, device=DEV, requires_grad=True)
+    rep, ii = c(x, epoch=15)
+    out = reconstruct(layers(rep), ii)
+    ref = layers(scatter_mean(x, ii, rep.size(0))).index_select(0, ii)
+    torch.testing.assert_close(out, ref, atol=1e-5, rtol=1e-4)
+    params = [x] + list(layers.parameters())
+    aa = torch.autograd.grad(out.square().sum(), params)
+    bb = torch.autograd.grad(ref.square().sum(), params)
+    for a, b in zip(aa, bb):
+        torch.testing.assert_close(a, b, atol=1e-5, rtol=1e-4)
+    # non-default stream
+    x = torch.randn(67, 33, device=DEV)
+    w = torch.randn(33, 8, device=DEV)
+    import compressgnn_runtime as native
+    ri, rc, ra = native.cluster_assign(x, w, 8, native.cluster_workspace(x, 8))
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        ii, cc, aa = native.cluster_assign(x, w, 8, native.cluster_workspace(x, 8))
+        yy = native.cluster_mean(x, ii, cc)
+    stream.synchronize()
+    assert torch.equal(ii, ri) and torch.equal(cc, rc) and aa == ra
+    torch.testing.assert_close(yy, scatter_mean(x, ri, ra + 1), atol=1e-5, rtol=1e-4)
+    # legacy entry
+    a = Compressgnn_Cluster(7, 4, device=DEV)
+    x = torch.randn(10, 7, device=DEV, requires_grad=True)
+    y, ii, active = Compressgnn_Cluster_Function.apply(x, a.random_vectors, 4, True)
+    ref = scatter_mean(x, ii, active + 1)
+    torch.testing.assert_close(y, ref, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(torch.autograd.grad(y.sum(), x)[0], torch.autograd.grad(ref.sum(), x)[0],
+                               atol=1e-5, rtol=1e-4)
+    with pytest.raises(RuntimeError):
+        native.cluster_assign(x, torch.randn(7, 3, device=DEV), 4, native.cluster_workspace(x, 4))
