@@ -1,0 +1,419 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+One "step" = one compressed propagation forward + backward (the 4-stage chain and its
+transpose) at F=128 over the C1 workload: a seeded copy-model web graph with 325,557
+vertices and about 3.2 M directed edges (+ self loops, symmetric normalisation),
+compressed by the batch pair merger and the saving/depth filters, fp32 N(0,1) features
+resident in HBM.  Prints ONE JSON line:
+
+  value        achieved HBM GB/s of a step = algorithmic bytes of the step / time per step
+  ms_per_step  milliseconds per forward+backward propagation
+  roofline     the dominant kernel (the fused vertex stage of the forward pass), timed with
+               HIP events inside the timed region
+  cpu_baseline the same step on the host cores (the reference's own CPU operator when
+               oracle/_ref is built, else the C oracle), timed in this run
+  detail       per-stage times, plain-CSR comparison, cluster + reconstruct times (C3)
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cluster] [--skip-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "compressgnn_amd")
+for p in (ROOT, PKG, os.path.join(PKG, "layer"), os.path.join(PKG, "loader")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0
+C1_VERTICES, C1_AVG_DEGREE, C1_COPY_PROB, C1_SEED = 325557, 9.8, 0.7, 1
+C3_NODES, C3_F, C3_H, C3_OUT, C3_CENTRES = 2449029, 100, 16, 256, 47
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def block_bytes(rowptr, col, ncols, F, acc, elt=4):
+    """Algorithmic bytes of one CSR product: indices + values (8 B per non-zero), row
+    pointers, every gathered input row once, every non-empty output row once (twice when
+    accumulating onto an existing output)."""
+    rowptr = np.asarray(rowptr)
+    col = np.asarray(col)
+    nnz = int(col.shape[0])
+    rows = int(rowptr.shape[0] - 1)
+    touched = int(np.unique(col).shape[0]) if nnz else 0
+    nonempty = int(np.count_nonzero(np.diff(rowptr)))
+    return dict(nnz=nnz, rows=rows, cols_touched=touched, rows_nonempty=nonempty,
+                bytes=8 * nnz + 4 * (rows + 1) + elt * F * touched + elt * F * nonempty * (1 + acc),
+                bytes_effective=8 * nnz + 4 * (rows + 1) + elt * F * nnz + elt * F * nonempty * (1 + acc),
+                flops=2 * nnz * F)
+
+
+def fused_bytes(b0, b1, rows, F, elt=4):
+    """The fused vertex stage: both blocks' indices and gathered rows, every output row
+    written exactly once, nothing read back."""
+    return (8 * (b0["nnz"] + b1["nnz"]) + 2 * 4 * (rows + 1) + elt * F * (b0["cols_touched"] + b1["cols_touched"])
+            + elt * F * rows)
+
+
+def graph_accounting(graph, F):
+    """Per-stage algorithmic bytes and flops of forward and backward propagation."""
+    def csr(g):
+        rp, ci, _ = g.csr()
+        return rp.cpu().numpy(), ci.cpu().numpy(), g.sparse_size(1)
+
+    def csc(g):
+        cp, row, _ = g.csc()
+        return cp.cpu().numpy(), row.cpu().numpy(), g.sparse_size(0)
+
+    V = graph.v2v_graph.sparse_size(0)
+    acct = {}
+    acct["fwd.rules"] = block_bytes(*csr(graph.r2v_graph), F, 0)
+    for i, g in enumerate(graph.r2r_graph):
+        acct["fwd.level%d" % i] = block_bytes(*csr(g), F, 1)
+    b0, b1 = block_bytes(*csr(graph.v2r_graph), F, 0), block_bytes(*csr(graph.v2v_graph), F, 1)
+    acct["fwd.final"] = dict(nnz=b0["nnz"] + b1["nnz"], bytes=fused_bytes(b0, b1, V, F),
+                             bytes_two_pass=b0["bytes"] + b1["bytes"], flops=b0["flops"] + b1["flops"])
+    acct["bwd.rules"] = block_bytes(*csc(graph.v2r_graph), F, 0)
+    for i, g in enumerate(graph.r2r_graph):
+        acct["bwd.level%d" % i] = block_bytes(*csc(g), F, 1)
+    b0, b1 = block_bytes(*csc(graph.r2v_graph), F, 0), block_bytes(*csc(graph.v2v_graph), F, 1)
+    acct["bwd.final"] = dict(nnz=b0["nnz"] + b1["nnz"], bytes=fused_bytes(b0, b1, V, F),
+                             bytes_two_pass=b0["bytes"] + b1["bytes"], flops=b0["flops"] + b1["flops"])
+    return acct
+
+
+def build_c1(F):
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    t0 = time.time()
+    v, e = off.gen_copy_model(C1_VERTICES, C1_AVG_DEGREE, C1_COPY_PROB, C1_SEED)
+    V = len(v) - 1
+    mask = np.zeros(V, dtype=bool)
+    data = CompressgnnData(np.zeros((V, 1), np.float32), (v, e), np.zeros(V, np.int64), mask, mask, mask,
+                           add_self_loop=True, normalize=True, graph_type="csr", max_depth=3, min_edge=1000000,
+                           threshold=16, min_pair_frequency=16, compression_rounds=12)
+    log("[bench] C1 graph: V=%d E=%d -> rules=%d compressed edges=%d levels=%d (%.1fs)" % (
+        V, len(e), data.rule_cnt, data.edge_cnt, data.edge_index.step, time.time() - t0))
+    return data, (v, e)
+
+
+def time_loop(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def stage_means(times):
+    agg = {}
+    for name, ms in times:
+        agg.setdefault(name, []).append(ms)
+    return {k: float(np.mean(v)) for k, v in agg.items()}
+
+
+def cpu_propagate_baseline(graph, x_np, g_np, iters=10):
+    """Forward + backward of the same step on the host cores: the reference's CPU
+    spmm_func ("rowbalance") when oracle/_ref is built, else the C oracle with OpenMP."""
+    import torch
+    def csr(g):
+        rp, ci, val = g.csr()
+        return rp.cpu(), ci.cpu(), val.cpu()
+
+    def csc(g):
+        cp, row, val = g.csc()
+        return cp.cpu(), row.cpu(), val.cpu()
+
+    fwd = dict(v2v=csr(graph.v2v_graph), v2r=csr(graph.v2r_graph), r2v=csr(graph.r2v_graph),
+               r2r=[csr(g) for g in graph.r2r_graph])
+    bwd = dict(v2v_t=csc(graph.v2v_graph), v2r_t=csc(graph.v2r_graph), r2v_t=csc(graph.r2v_graph),
+               r2r_t=[csc(g) for g in graph.r2r_graph])
+    cores = os.cpu_count() or 1
+    threads = min(16, cores)
+    kind = "port"
+    try:
+        sys.path.insert(0, os.path.join(ROOT, "oracle", "_ref"))
+        import compressgnn_runtime_ref as ref
+        kind = "reference"
+    except Exception as exc:  # not built on this box
+        log("[bench] oracle/_ref not available (%s); timing the C oracle instead" % exc)
+        ref = None
+    if ref is not None:
+        torch.set_num_threads(threads)
+        xt, gt = torch.from_numpy(x_np), torch.from_numpy(g_np)
+
+        def step():
+            ro = ref.spmm_func(*fwd["r2v"], xt, "rowbalance", None)
+            for lv in fwd["r2r"]:
+                ro = ref.spmm_func(*lv, ro, "rowbalance", ro)
+            out = ref.spmm_func(*fwd["v2r"], ro, "rowbalance", None)
+            out = ref.spmm_func(*fwd["v2v"], xt, "rowbalance", out)
+            rg = ref.spmm_func(*bwd["v2r_t"], gt, "rowbalance", None)
+            for lv in reversed(bwd["r2r_t"]):
+                rg = ref.spmm_func(*lv, rg, "rowbalance", rg)
+            gx = ref.spmm_func(*bwd["v2v_t"], gt, "rowbalance", None)
+            gx = ref.spmm_func(*bwd["r2v_t"], rg, "rowbalance", gx)
+            return out, gx
+    else:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+        npf = lambda blk: tuple(t.numpy() for t in blk)
+        fwd_np = dict(v2v=npf(fwd["v2v"]), v2r=npf(fwd["v2r"]), r2v=npf(fwd["r2v"]), r2r=[npf(b) for b in fwd["r2r"]])
+        bwd_np = dict(v2v_t=npf(bwd["v2v_t"]), v2r_t=npf(bwd["v2r_t"]), r2v_t=npf(bwd["r2v_t"]),
+                      r2r_t=[npf(b) for b in bwd["r2r_t"]])
+
+        def step():
+            return (oracle.compress_spmm_forward(fwd_np, x_np, threads),
+                    oracle.compress_spmm_backward(bwd_np, g_np, threads))
+    step()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        out = step()
+    ms = (time.perf_counter() - t0) / iters * 1e3
+    return ms, threads, cores, kind, out
+
+
+def bench_cluster(torch, steps, detail):
+    """C3: cluster (assign + members + mean) -> Linear 100->256 on representatives ->
+    reconstruct(bias, ReLU), forward and backward, per-operator times."""
+    import compressgnn_runtime as rt
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    centres = torch.randn(C3_CENTRES, C3_F, device=dev, generator=gen) * 2.0
+    which = torch.randint(0, C3_CENTRES, (C3_NODES,), device=dev, generator=gen)
+    x = centres.index_select(0, which) + torch.randn(C3_NODES, C3_F, device=dev, generator=gen)
+    del which
+    planes = torch.randn(C3_F, C3_H, device=dev, generator=gen)
+    weight = (torch.rand(C3_OUT, C3_F, device=dev, generator=gen) * 2 - 1) / (C3_F ** 0.5)
+    bias = (torch.rand(C3_OUT, device=dev, generator=gen) * 2 - 1) / (C3_F ** 0.5)
+    ws = rt.cluster_workspace(x, C3_H)
+
+    def timed(fn, reps=steps):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            out = fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps, out
+
+    N, F, Fo = C3_NODES, C3_F, C3_OUT
+    t_assign, (ids, counts, active) = timed(lambda: rt.cluster_assign(x, planes, C3_H, ws))
+    groups = active + 1
+    t_members, members = timed(lambda: rt.cluster_members(ids, groups))
+    t_mean, reps = timed(lambda: rt.cluster_mean(x, ids, counts, members))
+    t_linear, hidden = timed(lambda: torch.nn.functional.linear(reps, weight))
+    t_recon, out = timed(lambda: rt.cluster_reconstruct(hidden, ids, bias, True))
+    grad_out = torch.randn(N, Fo, device=dev, generator=gen)
+    t_recon_bwd, hidden_grad = timed(lambda: rt.cluster_reconstruct_backward(grad_out, ids, out, groups, True, members))
+    t_linear_bwd, reps_grad = timed(lambda: hidden_grad @ weight)
+    t_mean_bwd, dx = timed(lambda: rt.cluster_mean_backward(reps_grad, ids, counts))
+    gb = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    C = groups
+    ops = {
+        "assign": dict(ms=t_assign, bytes=4 * N * F + 4 * F * C3_H + 8 * N),
+        "members": dict(ms=t_members, bytes=8 * N + 8 * N + 4 * C),
+        "mean": dict(ms=t_mean, bytes=4 * N * F + 8 * N + 4 * C * F),
+        "reconstruct": dict(ms=t_recon, bytes=4 * C * Fo + 8 * N + 4 * Fo + 4 * N * Fo),
+        "reconstruct_backward": dict(ms=t_recon_bwd, bytes=2 * 4 * N * Fo + 8 * N + 4 * C * Fo),
+        "mean_backward": dict(ms=t_mean_bwd, bytes=4 * C * F + 8 * N + 4 * N * F),
+    }
+    for k, v in ops.items():
+        v["GBps"] = gb(v["bytes"], v["ms"])
+        v["frac_of_hbm_peak"] = v["GBps"] / HBM_PEAK_GBPS
+    reuse = t_mean + t_linear + t_recon + t_recon_bwd + t_linear_bwd + t_mean_bwd
+    refresh = reuse + t_assign + t_members
+    detail["cluster_reconstruct_C3"] = dict(
+        nodes=N, in_features=F, bits=C3_H, out_features=Fo, active_clusters=int(active), ops=ops,
+        linear_ms=t_linear, linear_backward_ms=t_linear_bwd,
+        fwd_bwd_ms_refresh_epoch=refresh, fwd_bwd_ms_reuse_epoch=reuse,
+        fwd_bwd_ms_per_epoch_refresh_interval_1=refresh,
+        fwd_bwd_ms_per_epoch_refresh_interval_5=(refresh + 4 * reuse) / 5)
+    log("[bench] C3 cluster+reconstruct: " + ", ".join("%s %.3f ms (%.0f GB/s)" % (k, v["ms"], v["GBps"])
+                                                        for k, v in ops.items()))
+    return x, planes
+
+
+def cpu_cluster_baseline(x, planes, detail, sample=200000):
+    """assign + mean + reconstruct(bias, relu) + their gradients on a bounded sample of
+    the C3 rows on the host (C oracle)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle
+    xs = x[:sample].cpu().numpy()
+    pl = planes.cpu().numpy()
+    rng = np.random.default_rng(0)
+    threads = min(16, os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    ids, counts, active = oracle.assign(xs, pl, C3_H)
+    t1 = time.perf_counter()
+    reps = oracle.cluster_mean(xs, ids, counts)
+    hidden = rng.standard_normal((active + 1, C3_OUT)).astype(np.float32)
+    bias = rng.standard_normal(C3_OUT).astype(np.float32)
+    t2 = time.perf_counter()
+    out = oracle.reconstruct(hidden, ids, bias, True, threads)
+    t3 = time.perf_counter()
+    go = rng.standard_normal(out.shape).astype(np.float32)
+    t4 = time.perf_counter()
+    oracle.reconstruct_backward(go, ids, out, active + 1, True)
+    t5 = time.perf_counter()
+    oracle.cluster_mean_backward(reps, ids, counts, threads)
+    t6 = time.perf_counter()
+    detail["cluster_reconstruct_cpu_sample"] = dict(
+        rows=sample, kind="port", threads=threads, assign_ms=(t1 - t0) * 1e3, mean_ms=(t2 - t1) * 1e3,
+        reconstruct_ms=(t3 - t2) * 1e3, reconstruct_backward_ms=(t5 - t4) * 1e3, mean_backward_ms=(t6 - t5) * 1e3)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--features", type=int, default=128)
+    ap.add_argument("--skip-cluster", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--sweep", action="store_true", help="also time F in {16, 64, 256, 512} (C2)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path uses no "
+                 "collectives, see DESIGN.md for how it would shard)" % args.gpus)
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    import compressgnn_runtime as rt
+    from CompressgnnSPMM import compress_spmm  # noqa: F401  (the layer path uses the same plan)
+
+    F = args.features
+    dev = torch.device("cuda:0")
+    data, (v_raw, e_raw) = build_c1(F)
+    graph = data.edge_index
+    acct = graph_accounting(graph, F)
+    data.to(dev)
+    plan = graph.plan()
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    x = torch.randn(C1_VERTICES, F, device=dev, generator=gen)
+    g = torch.randn(C1_VERTICES, F, device=dev, generator=gen)
+
+    def step():
+        out = plan.forward(x)
+        gx = plan.backward(g)
+        return out, gx
+
+    # the timed region: K steps, one pair of HIP events around the dominant kernel
+    plan.timed_stages = ["fwd.final"]
+    ms_step = time_loop(step, args.steps, args.warmup, torch)
+    dom = stage_means(plan.take_stage_times())["fwd.final"]
+    # second pass with every stage timed (adds event overhead; not the headline)
+    plan.timed_stages = ["*"]
+    time_loop(step, min(args.steps, 20), 1, torch)
+    stages = stage_means(plan.take_stage_times())
+    plan.timed_stages = []
+
+    step_bytes = sum(a["bytes"] for a in acct.values())
+    step_flops = sum(a["flops"] for a in acct.values())
+    value = step_bytes / (ms_step * 1e-3) / 1e9
+    dom_bytes = acct["fwd.final"]["bytes"]
+    dom_gbps = dom_bytes / (dom * 1e-3) / 1e9
+
+    detail = dict(
+        graph=dict(vertices=C1_VERTICES, edges=int(len(e_raw)), edges_with_self_loops=int(len(e_raw)) + C1_VERTICES,
+                   rules=int(data.rule_cnt), compressed_edges=int(data.edge_cnt), levels=int(graph.step)),
+        step_bytes=step_bytes, step_gflop=step_flops / 1e9, gflops=step_flops / (ms_step * 1e-3) / 1e9,
+        stages={k: dict(ms=stages.get(k), bytes=a["bytes"], nnz=a["nnz"],
+                        GBps=(a["bytes"] / (stages[k] * 1e-3) / 1e9) if stages.get(k) else None)
+                for k, a in acct.items()},
+    )
+
+    # forward-only and backward-only times, and the plain (uncompressed) CSR product
+    detail["forward_ms"] = time_loop(lambda: plan.forward(x), args.steps, 2, torch)
+    detail["backward_ms"] = time_loop(lambda: plan.backward(g), args.steps, 2, torch)
+    import compressgnn_offline as off
+    v2, e2 = off.add_self_loop_csr(v_raw, e_raw)
+    d = off.get_norm_degree(e2, C1_VERTICES)
+    src = np.repeat(np.arange(C1_VERTICES), np.diff(v2))
+    w = (d[src] * d[e2]).astype(np.float32)
+    cp, row, wt = off.csr_transpose(v2, e2, w, C1_VERTICES)
+    plain_t = rt.DeviceCsr(torch.from_numpy(cp), torch.from_numpy(row), torch.from_numpy(wt), C1_VERTICES,
+                           C1_VERTICES, dev)
+    plain = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(e2), torch.from_numpy(w), C1_VERTICES,
+                         C1_VERTICES, dev)
+    pb_f, pb_b = block_bytes(cp, row, C1_VERTICES, F, 0), block_bytes(v2, e2, C1_VERTICES, F, 0)
+    for name in ("rowbalance", "nnzbalance"):
+        f_ms = time_loop(lambda: plain_t.spmm(x, None, name), args.steps, 2, torch)
+        b_ms = time_loop(lambda: plain.spmm(g, None, name), args.steps, 2, torch)
+        detail["plain_csr_%s" % name] = dict(forward_ms=f_ms, backward_ms=b_ms,
+                                             forward_GBps=pb_f["bytes"] / (f_ms * 1e-3) / 1e9,
+                                             backward_GBps=pb_b["bytes"] / (b_ms * 1e-3) / 1e9,
+                                             forward_bytes=pb_f["bytes"], backward_bytes=pb_b["bytes"])
+    # parity of the measured configuration: compressed == plain within tolerance
+    out, gx = step()
+    ref_out = plain_t.spmm(x, None, "rowbalance")
+    err = (out - ref_out).abs().max().item()
+    detail["max_abs_diff_vs_plain_csr"] = err
+
+    if args.sweep:
+        sweep = {}
+        for Fs in (16, 64, 256, 512):
+            xs = torch.randn(C1_VERTICES, Fs, device=dev, generator=gen)
+            gs = torch.randn(C1_VERTICES, Fs, device=dev, generator=gen)
+            ms = time_loop(lambda: (plan.forward(xs), plan.backward(gs)), args.steps, 2, torch)
+            a = graph_accounting(graph.to("cpu") if False else graph, Fs)
+            nbytes = sum(t["bytes"] for t in a.values())
+            sweep[str(Fs)] = dict(ms_per_step=ms, bytes=nbytes, GBps=nbytes / (ms * 1e-3) / 1e9)
+            del xs, gs
+        detail["feature_sweep_C2"] = sweep
+
+    cpu = None
+    if not args.skip_cpu:
+        x_np, g_np = x.cpu().numpy(), g.cpu().numpy()
+        ms_cpu, threads, cores, kind, (out_cpu, gx_cpu) = cpu_propagate_baseline(graph, x_np, g_np)
+        out_cpu = out_cpu.numpy() if hasattr(out_cpu, "numpy") else out_cpu
+        detail["max_abs_diff_vs_cpu_baseline"] = float(np.abs(out.cpu().numpy() - out_cpu).max())
+        cpu = dict(value=step_bytes / (ms_cpu * 1e-3) / 1e9, unit="GB/s", ms_per_step=ms_cpu, cores=threads,
+                   host_cores=cores, kind=kind,
+                   sample="the whole C1 step (forward + backward propagation, F=%d), 1 warm-up + 10 iterations" % F)
+        log("[bench] CPU baseline (%s, %d threads): %.1f ms per step" % (kind, threads, ms_cpu))
+
+    del plain, plain_t
+    if not args.skip_cluster:
+        torch.cuda.empty_cache()
+        xc, planes = bench_cluster(torch, max(3, min(args.steps, 10)), detail)
+        if not args.skip_cpu:
+            cpu_cluster_baseline(xc, planes, detail)
+
+    result = {
+        "metric": "compressed_propagate_fwd_bwd_hbm_GBps_F%d" % F,
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "C1: copy-model web graph, 325,557 vertices / %d directed edges (+ self loops, "
+                               "sym-norm), compressed propagation forward + backward, F=%d fp32" % (len(e_raw), F),
+                   "rules": int(data.rule_cnt), "levels": int(graph.step)},
+        "frac_of_hbm_peak": value / HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "spmm_pair_kernel (forward vertex stage: v2r + v2v fused)",
+                     "achieved": dom_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom_gbps / HBM_PEAK_GBPS,
+                     "traffic": None, "ms": dom, "bytes": dom_bytes},
+        "cpu_baseline": cpu,
+        "detail": detail,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

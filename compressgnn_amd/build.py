@@ -104,7 +104,7 @@ def build_runtime():
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared",
            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=compressgnn_runtime",
            "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
-           "-Wno-deprecated-declarations"] + inc + [
+           "-Wno-deprecated-declarations", "-Wno-unused-result"] + inc + [
            os.path.join(CSRC, "torch_binding.cpp"), "-o", out,
            "-L", torch_lib, "-L", LIB_DIR, "-L", "/opt/rocm/lib",
            "-Wl,-rpath," + torch_lib, "-Wl,-rpath,$ORIGIN/lib", "-Wl,-rpath,/opt/rocm/lib",

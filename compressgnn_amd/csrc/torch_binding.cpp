@@ -5,8 +5,9 @@
 // (include/compressgnn_abi.h); torch supplies tensors, the caching allocator and the
 // current stream.  There is no CPU implementation behind these operators: CPU tensors
 // are rejected with an error.
-#include <ATen/hip/HIPContext.h>
-#include <c10/hip/HIPGuard.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
 #include <map>
@@ -26,7 +27,7 @@ void ok(int rc, const char *what) {
 }
 
 cgnn_stream_t current_stream(const Tensor &t) {
-    return reinterpret_cast<cgnn_stream_t>(at::hip::getCurrentHIPStream(t.device().index()).stream());
+    return reinterpret_cast<cgnn_stream_t>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream());
 }
 
 int dtype_code(const Tensor &t) {
@@ -91,7 +92,7 @@ std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Ten
     blk->seg_nnz = (int32_t)seg_nnz;
     const int64_t lim = (int64_t)INT32_MAX - 65536;
     TORCH_CHECK(rows < lim && cols < lim && blk->nnz < lim, "block exceeds the int32 index range of the kernels");
-    c10::hip::HIPGuard guard(device);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(device);
     Tensor rp = rowptr.to(device).contiguous();
     Tensor ci = col.to(device).contiguous();
     auto i32 = torch::TensorOptions().device(device).dtype(torch::kInt32);
@@ -146,7 +147,7 @@ Tensor block_spmm(DeviceCsr &A, const Tensor &mat, c10::optional<Tensor> optiona
     TORCH_CHECK(mat.dim() == 2, "mat must be a matrix");
     TORCH_CHECK(mat.size(0) == A.cols, "mat has ", mat.size(0), " rows, the block has ", A.cols, " columns");
     TORCH_CHECK(!A.val.defined() || A.val.scalar_type() == mat.scalar_type(), "value and mat must have the same dtype");
-    c10::hip::HIPGuard guard(mat.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(mat.device());
     const int64_t F = mat.size(1);
     const int dtype = dtype_code(mat);
     Tensor out;
@@ -190,6 +191,55 @@ Tensor spmm_func(Tensor vlist, Tensor elist, Tensor value, Tensor mat, std::stri
 
 // ------------------------------------------------------- compressed propagation ----
 
+// Optional per-stage timing with HIP events on the stream the kernels run on.  Events
+// are recorded only around the stages named in `timed` ("*" = all), so a timed region
+// can carry one pair of events per step without disturbing the rest.
+struct StageTimer {
+    struct Rec {
+        std::string name;
+        hipEvent_t begin, end;
+    };
+    std::vector<std::string> timed;
+    std::vector<Rec> recs;
+
+    bool wants(const std::string &name) const {
+        for (auto &t : timed)
+            if (t == "*" || t == name) return true;
+        return false;
+    }
+    int open(const std::string &name, hipStream_t stream) {
+        if (!wants(name)) return -1;
+        Rec r{name, nullptr, nullptr};
+        TORCH_CHECK(hipEventCreate(&r.begin) == hipSuccess && hipEventCreate(&r.end) == hipSuccess, "hipEventCreate failed");
+        TORCH_CHECK(hipEventRecord(r.begin, stream) == hipSuccess, "hipEventRecord failed");
+        recs.push_back(r);
+        return (int)recs.size() - 1;
+    }
+    void close(int id, hipStream_t stream) {
+        if (id >= 0) TORCH_CHECK(hipEventRecord(recs[id].end, stream) == hipSuccess, "hipEventRecord failed");
+    }
+    // (stage, milliseconds) of every recorded interval; call after the stream is idle.
+    std::vector<std::pair<std::string, double>> take() {
+        std::vector<std::pair<std::string, double>> out;
+        for (auto &r : recs) {
+            float ms = 0;
+            TORCH_CHECK(hipEventSynchronize(r.end) == hipSuccess, "hipEventSynchronize failed");
+            TORCH_CHECK(hipEventElapsedTime(&ms, r.begin, r.end) == hipSuccess, "hipEventElapsedTime failed");
+            out.emplace_back(r.name, (double)ms);
+            hipEventDestroy(r.begin);
+            hipEventDestroy(r.end);
+        }
+        recs.clear();
+        return out;
+    }
+    ~StageTimer() {
+        for (auto &r : recs) {
+            hipEventDestroy(r.begin);
+            hipEventDestroy(r.end);
+        }
+    }
+};
+
 // The device form of a CompressGraph (loader/compress_graph.py:6-43 of the reference):
 // the three vertex/rule blocks, the rule levels and their transposes.
 struct PropagationPlan {
@@ -198,44 +248,61 @@ struct PropagationPlan {
     int64_t V = 0, R = 0;
     bool fuse_final = true;  // last two stages in one pass (cgnn_spmm_pair)
     int kernel = CGNN_SPMM_AUTO;
+    StageTimer timer;
 };
 
-Tensor final_stage(PropagationPlan &p, DeviceCsr &from_rules, const Tensor &rule_x, DeviceCsr &from_vertices,
-                   const Tensor &x) {
+Tensor timed_spmm(PropagationPlan &p, const std::string &stage, DeviceCsr &A, const Tensor &mat,
+                  c10::optional<Tensor> out) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(current_stream(mat));
+    const int id = p.timer.open(stage, stream);
+    Tensor r = block_spmm(A, mat, out, p.kernel);
+    p.timer.close(id, stream);
+    return r;
+}
+
+Tensor final_stage(PropagationPlan &p, const std::string &prefix, DeviceCsr &from_rules, const Tensor &rule_x,
+                   DeviceCsr &from_vertices, const Tensor &x) {
     const int64_t F = x.size(1);
     if (p.fuse_final) {
         Tensor out = torch::empty({from_vertices.rows, F}, x.options());
         if (out.numel() == 0) return out;
+        hipStream_t stream = reinterpret_cast<hipStream_t>(current_stream(x));
+        const int id = p.timer.open(prefix + "final", stream);
         cgnn_csr a0 = from_rules.view(), a1 = from_vertices.view();
         ok(cgnn_spmm_pair(&a0, rule_x.data_ptr(), &a1, x.data_ptr(), dtype_code(x), out.data_ptr(), F,
                           current_stream(x)),
            "spmm_pair");
+        p.timer.close(id, stream);
         return out;
     }
-    Tensor out = block_spmm(from_rules, rule_x, c10::nullopt, p.kernel);
-    return block_spmm(from_vertices, x, out, p.kernel);
+    Tensor out = timed_spmm(p, prefix + "from_rules", from_rules, rule_x, c10::nullopt);
+    return timed_spmm(p, prefix + "from_vertices", from_vertices, x, out);
 }
 
-// layer/CompressgnnSPMM.py:43-62 of the reference.
+// layer/CompressgnnSPMM.py:43-62 of the reference.  Stage names: fwd.rules (r2v),
+// fwd.level<i>, fwd.final (v2r + v2v fused) or fwd.from_rules / fwd.from_vertices.
 Tensor propagate_forward(PropagationPlan &p, Tensor x) {
     require_gpu(x, "x");
     TORCH_CHECK(x.dim() == 2 && x.size(0) == p.V, "x must be [vertex_cnt, F]");
     x = x.contiguous();
-    c10::hip::HIPGuard guard(x.device());
-    Tensor rule_out = block_spmm(*p.r2v, x, c10::nullopt, p.kernel);
-    for (auto &level : p.r2r) rule_out = block_spmm(*level, rule_out, rule_out, p.kernel);
-    return final_stage(p, *p.v2r, rule_out, *p.v2v, x);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    Tensor rule_out = timed_spmm(p, "fwd.rules", *p.r2v, x, c10::nullopt);
+    for (size_t i = 0; i < p.r2r.size(); ++i)
+        rule_out = timed_spmm(p, "fwd.level" + std::to_string(i), *p.r2r[i], rule_out, rule_out);
+    return final_stage(p, "fwd.", *p.v2r, rule_out, *p.v2v, x);
 }
 
-// layer/CompressgnnSPMM.py:65-86 (the working branch, lines 80-85).
+// layer/CompressgnnSPMM.py:65-86 (the working branch, lines 80-85).  Stage names as in
+// forward with the prefix bwd.
 Tensor propagate_backward(PropagationPlan &p, Tensor grad) {
     require_gpu(grad, "grad");
     TORCH_CHECK(grad.dim() == 2 && grad.size(0) == p.V, "grad must be [vertex_cnt, F]");
     grad = grad.contiguous();
-    c10::hip::HIPGuard guard(grad.device());
-    Tensor rule_g = block_spmm(*p.v2r_t, grad, c10::nullopt, p.kernel);
-    for (auto it = p.r2r_t.rbegin(); it != p.r2r_t.rend(); ++it) rule_g = block_spmm(**it, rule_g, rule_g, p.kernel);
-    return final_stage(p, *p.r2v_t, rule_g, *p.v2v_t, grad);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
+    Tensor rule_g = timed_spmm(p, "bwd.rules", *p.v2r_t, grad, c10::nullopt);
+    for (size_t i = p.r2r_t.size(); i-- > 0;)
+        rule_g = timed_spmm(p, "bwd.level" + std::to_string(i), *p.r2r_t[i], rule_g, rule_g);
+    return final_stage(p, "bwd.", *p.r2v_t, rule_g, *p.v2v_t, grad);
 }
 
 // ---------------------------------------------------- transformation compression ----
@@ -265,7 +332,7 @@ void check_count(const Tensor &count, torch::Device device) {
 // [bucket counts int32[2^bits], prefix int32[2^bits], scan scratch uint8[...]].
 std::vector<Tensor> cluster_workspace(Tensor input, int64_t bits) {
     check_float(input);
-    c10::hip::HIPGuard guard(input.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const int n = bucket_size(bits);
     auto ints = input.options().dtype(torch::kInt32);
     return {torch::empty({n}, ints), torch::empty({n}, ints),
@@ -277,7 +344,7 @@ std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, 
                                                    std::vector<Tensor> workspace) {
     check_float(input);
     check_float(planes);
-    c10::hip::HIPGuard guard(input.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const int n = bucket_size(bits);
     TORCH_CHECK(planes.device() == input.device() && planes.scalar_type() == input.scalar_type() &&
                     planes.size(0) == input.size(1) && planes.size(1) == bits,
@@ -334,7 +401,7 @@ std::vector<Tensor> cluster_members(Tensor index, int64_t groups) {
     TORCH_CHECK(index.is_cuda(), "index must be a GPU tensor");
     check_index(index, index.device());
     TORCH_CHECK(groups >= 1, "groups must be positive");
-    c10::hip::HIPGuard guard(index.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(index.device());
     const int64_t N = index.numel();
     auto i32 = index.options().dtype(torch::kInt32);
     Tensor offsets = torch::empty({groups + 1}, i32), perm = torch::empty({N}, i32), sorted = torch::empty({N}, i32);
@@ -368,7 +435,7 @@ Tensor cluster_mean(Tensor input, Tensor index, Tensor count, c10::optional<std:
     check_index(index, input.device());
     check_count(count, input.device());
     TORCH_CHECK(index.numel() == input.size(0), "Input/index length mismatch");
-    c10::hip::HIPGuard guard(input.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const int64_t N = input.size(0), F = input.size(1), groups = count.numel();
     if (input.numel() == 0) return torch::zeros({groups, F}, input.options());
     auto m = members_or_build(members, index, groups);
@@ -388,7 +455,7 @@ Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count) {
     check_index(index, grad.device());
     check_count(count, grad.device());
     TORCH_CHECK(grad.size(0) == count.numel(), "Gradient/count shape mismatch");
-    c10::hip::HIPGuard guard(grad.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
     Tensor out = torch::empty({index.numel(), grad.size(1)}, grad.options());
     if (out.numel() == 0) return out;
     ok(cgnn_cluster_mean_backward(index.numel(), grad.size(1), count.numel(), dtype_code(grad), grad.data_ptr(),
@@ -406,7 +473,7 @@ Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias
         TORCH_CHECK(bias->device() == reps.device() && bias->scalar_type() == reps.scalar_type() && bias->dim() == 1 &&
                         bias->numel() == reps.size(1) && bias->is_contiguous(),
                     "Invalid reconstruction bias");
-    c10::hip::HIPGuard guard(reps.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(reps.device());
     Tensor out = torch::empty({index.numel(), reps.size(1)}, reps.options());
     if (out.numel() == 0) return out;
     ok(cgnn_reconstruct(index.numel(), reps.size(1), reps.size(0), dtype_code(reps), reps.data_ptr(),
@@ -425,7 +492,7 @@ Tensor cluster_reconstruct_backward(Tensor grad, Tensor index, Tensor output, in
     TORCH_CHECK(groups >= 0 && output.sizes() == grad.sizes() && output.device() == grad.device() &&
                     output.scalar_type() == grad.scalar_type() && index.numel() == grad.size(0),
                 "Invalid reconstruction gradient");
-    c10::hip::HIPGuard guard(grad.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
     const int64_t N = grad.size(0), F = grad.size(1);
     if (grad.numel() == 0 || groups == 0) return torch::zeros({groups, F}, grad.options());
     auto m = members_or_build(members, index, groups);
@@ -496,6 +563,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def_property("method",
                       [](PropagationPlan &p) { return p.kernel == CGNN_SPMM_ROW ? "rowbalance" : p.kernel == CGNN_SPMM_NNZ ? "nnzbalance" : "auto"; },
                       [](PropagationPlan &p, std::string mth) { p.kernel = kernel_of_method(mth); })
+        .def_property("timed_stages", [](PropagationPlan &p) { return p.timer.timed; },
+                      [](PropagationPlan &p, std::vector<std::string> names) { p.timer.timed = names; })
+        .def("take_stage_times", [](PropagationPlan &p) { return p.timer.take(); })
+        .def_readonly("v2v", &PropagationPlan::v2v)
+        .def_readonly("v2r", &PropagationPlan::v2r)
+        .def_readonly("r2v", &PropagationPlan::r2v)
+        .def_readonly("r2r", &PropagationPlan::r2r)
+        .def_readonly("v2v_t", &PropagationPlan::v2v_t)
+        .def_readonly("v2r_t", &PropagationPlan::v2r_t)
+        .def_readonly("r2v_t", &PropagationPlan::r2v_t)
+        .def_readonly("r2r_t", &PropagationPlan::r2r_t)
         .def("forward", &propagate_forward)
         .def("backward", &propagate_backward);
 }
