@@ -17,7 +17,7 @@ SPMM_AUTO, SPMM_ROW, SPMM_NNZ = 0, 1, 2
 
 EXPORTS = [
     "cgnn_last_error", "cgnn_version",
-    "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_pair",
+    "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
     "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_hash", "cgnn_lsh_scan", "cgnn_lsh_finish",
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
@@ -143,13 +143,15 @@ def spmm(A, X, Y=None, accumulate=False, kernel=SPMM_AUTO):
     return Y
 
 
-def spmm_pair(A0, X0, A1, X1, Y=None):
+def spmm_dual(A, split, X0, X1, Y=None, kernel=SPMM_AUTO):
+    """Y = A[:, :split] @ X0 + A[:, split:] @ X1 in one pass through cgnn_spmm_dual."""
     F = X0.shape[1]
     if Y is None:
-        Y = torch.empty((A0.rows, F), dtype=X0.dtype, device=X0.device)
-    s0, s1 = A0.struct(), A1.struct()
-    check(lib().cgnn_spmm_pair(ctypes.byref(s0), ptr(X0), ctypes.byref(s1), ptr(X1),
-                               dtype_code(X0.dtype), ptr(Y), i64(F), stream_of(X0)))
+        Y = torch.empty((A.rows, F), dtype=X0.dtype, device=X0.device)
+    ws, need = A.workspace(F, X0.dtype, kernel)
+    s = A.struct()
+    check(lib().cgnn_spmm_dual(ctypes.byref(s), i64(split), dtype_code(X0.dtype), ptr(X0), ptr(X1), ptr(Y),
+                               i64(F), ctypes.c_int(kernel), ptr(ws), ctypes.c_size_t(need), stream_of(X0)))
     return Y
 
 

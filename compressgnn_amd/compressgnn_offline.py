@@ -19,7 +19,7 @@ EXPORTS = [
     "cgnn_add_self_loop_csr", "cgnn_get_norm_degree", "cgnn_gcn_norm_csr_compress",
     "cgnn_csr_transpose", "cgnn_hybird_partition", "cgnn_topo_partition", "cgnn_gen_degree",
     "cgnn_filter_csr", "cgnn_depth_filter_csr", "cgnn_gen_vertex_order_csr", "cgnn_gen_vertex_order_csc",
-    "cgnn_compress_csr_batch", "cgnn_csr_row_stats", "cgnn_gen_chung_lu", "cgnn_gen_copy_model",
+    "cgnn_compress_csr_batch", "cgnn_csr_hstack", "cgnn_csr_row_stats", "cgnn_gen_chung_lu", "cgnn_gen_copy_model",
 ]
 
 _NP_TYPES = {0: np.int64, 1: np.float32, 2: np.int32}
@@ -217,6 +217,17 @@ def csr2coo(vlist, elist):
     vlist, elist = _i64(vlist), _i64(elist)
     src = np.repeat(np.arange(len(vlist) - 1, dtype=np.int64), np.diff(vlist))
     return src, elist.copy()
+
+
+def csr_hstack(a0, a1, col_offset):
+    """[A0 | A1] for two CSR triples (vlist, elist, value) with the same number of rows."""
+    v0, e0, w0 = _i64(a0[0]), _i64(a0[1]), _f32(a0[2])
+    v1, e1, w1 = _i64(a1[0]), _i64(a1[1]), _f32(a1[2])
+    if len(v0) != len(v1):
+        raise ValueError("csr_hstack: blocks must have the same number of rows")
+    (v, e, w), _ = _take(lib().cgnn_csr_hstack(ctypes.c_int64(len(v0) - 1), _p(v0), _p(e0), _p(w0), _p(v1), _p(e1),
+                                               _p(w1), ctypes.c_int64(col_offset)))
+    return v, e, w
 
 
 def csr_row_stats(vlist):

@@ -793,6 +793,37 @@ cgnn_arrays *cgnn_compress_csr_batch(int64_t V, const int64_t *vlist, const int6
     return guarded([&] { return compress_batch(V, vlist, elist, rounds, min_pair_frequency); });
 }
 
+cgnn_arrays *cgnn_csr_hstack(int64_t rows, const int64_t *vlist0, const int64_t *elist0, const float *value0,
+                             const int64_t *vlist1, const int64_t *elist1, const float *value1, int64_t col_offset) {
+    if (rows < 0 || !vlist0 || !vlist1) {
+        set_error("csr_hstack: bad arguments");
+        return nullptr;
+    }
+    return guarded([&] {
+        const i64 n0 = vlist0[rows], n1 = vlist1[rows];
+        std::vector<i64> ptr(rows + 1, 0), col;
+        std::vector<float> val;
+        col.reserve(n0 + n1);
+        val.reserve(n0 + n1);
+        for (i64 r = 0; r < rows; ++r) {
+            for (i64 e = vlist0[r]; e < vlist0[r + 1]; ++e) {
+                col.push_back(elist0[e]);
+                val.push_back(value0[e]);
+            }
+            for (i64 e = vlist1[r]; e < vlist1[r + 1]; ++e) {
+                col.push_back(elist1[e] + col_offset);
+                val.push_back(value1[e]);
+            }
+            ptr[r + 1] = (i64)col.size();
+        }
+        auto *out = new cgnn_arrays;
+        out->add(std::move(ptr));
+        out->add(std::move(col));
+        out->add(std::move(val));
+        return out;
+    });
+}
+
 int cgnn_csr_row_stats(int64_t rows, const int64_t *vlist, int64_t *max_row, int64_t hist[40]) {
     if (rows < 0 || !vlist) {
         set_error("csr_row_stats: bad arguments");

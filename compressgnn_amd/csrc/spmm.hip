@@ -3,10 +3,9 @@
 // Geometry shared by all kernels here.  A "lane group" of LPR consecutive lanes
 // (LPR a power of two, 4..64) owns one output row at a time; lane l of the group
 // holds VEC consecutive features starting at (tile*LPR + l)*VEC for TILES tiles, so a
-// group reads and writes LPR*VEC*sizeof(T) contiguous bytes per tile: 512 B per wave
-// instruction when VEC*sizeof(T) = 16 (global_load_dwordx4) and LPR*... covers a row.
-// Features beyond LPR*VEC*TILES are covered by blockIdx.y.  Index data are wave-uniform
-// when LPR == 64, so the compiler fetches them through the scalar unit.
+// group reads and writes LPR*VEC*sizeof(T) contiguous bytes per tile (512 B per wave
+// instruction when VEC*sizeof(T) = 16, i.e. global_load_dwordx4 on every lane).
+// Features beyond LPR*VEC*TILES are covered by blockIdx.y.
 //
 // Two schedules:
 //   * row schedule  -- a lane group per row, entries summed in ascending order; the
@@ -20,9 +19,16 @@
 //     carry row and added by spmm_fixup_kernel, which walks the carries of one row in
 //     ascending run order.  No atomics anywhere, so results are reproducible run to run.
 //
+// Modes: VAL (stored values), UNIT (all values 1), RELU_MASK (unit values, gathered
+// rows zeroed where a second matrix is <= 0), DUAL (columns below `split` gather from
+// X, the others from X1; the two partial sums are kept apart and combined as
+// (0 + sum1) + sum0, which is what two successive accumulating products give).
+//
 // X may alias Y when accumulating (rule levels are updated in place, reference
 // layer/CompressgnnSPMM.py:56-58), so X and Y carry no __restrict__; a row that is
 // written is never gathered in the same launch (levels only read earlier levels).
+#include <cstdlib>
+
 #include "common.h"
 
 namespace cgnn {
@@ -31,7 +37,7 @@ namespace {
 constexpr int kUnroll = 8;        // gathers in flight per lane and tile
 constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
 
-enum { MODE_VAL = 0, MODE_UNIT = 1, MODE_RELU_MASK = 2 };
+enum { MODE_VAL = 0, MODE_UNIT = 1, MODE_RELU_MASK = 2, MODE_DUAL = 3 };
 
 template <typename T, int VEC>
 struct alignas(sizeof(T) * VEC) Pack {
@@ -40,11 +46,12 @@ struct alignas(sizeof(T) * VEC) Pack {
 
 template <typename T>
 struct SpmmArgs {
-    const int32_t *__restrict__ rowptr;
-    const int32_t *__restrict__ colidx;
-    const int32_t *__restrict__ rowidx;
-    const T *__restrict__ val;
+    const int32_t *rowptr;
+    const int32_t *colidx;
+    const int32_t *rowidx;
+    const T *val;
     const T *X;   // gathered matrix (may alias Y)
+    const T *X1;  // MODE_DUAL: source of the columns >= split
     const T *M;   // MODE_RELU_MASK: rows of X are zeroed where M <= 0
     T *Y;
     int32_t *carry_row;  // [nseg] row a run carries into, or -1
@@ -54,6 +61,7 @@ struct SpmmArgs {
     int32_t nnz;
     int32_t nseg;
     int32_t seg_nnz;
+    int32_t split;
     int32_t accumulate;
 };
 
@@ -76,18 +84,50 @@ __device__ __forceinline__ void feature_offsets(int64_t F, int lane, int64_t fof
     }
 }
 
-template <typename T, int VEC, int TILES>
-__device__ __forceinline__ void zero_acc(Pack<T, VEC> acc[TILES]) {
+// Accumulators of one output row: one set, or two in MODE_DUAL.
+template <typename T, int VEC, int TILES, int MODE>
+struct Acc {
+    static constexpr int SETS = MODE == MODE_DUAL ? 2 : 1;
+    Pack<T, VEC> a[SETS][TILES];
+
+    __device__ __forceinline__ void clear() {
 #pragma unroll
-    for (int t = 0; t < TILES; ++t)
+        for (int s = 0; s < SETS; ++s)
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[t].v[i] = T(0);
-}
+            for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) a[s][t].v[i] = T(0);
+    }
+    // entry with gathered tiles x, value w, from source `src` (0 or 1)
+    __device__ __forceinline__ void add(const Pack<T, VEC> x[TILES], T w, int src) {
+        if constexpr (MODE == MODE_DUAL) {
+            if (src) {
+#pragma unroll
+                for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) a[1][t].v[i] = a[1][t].v[i] + x[t].v[i] * w;
+                return;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) a[0][t].v[i] = a[0][t].v[i] + x[t].v[i] * w;
+                else a[0][t].v[i] = a[0][t].v[i] + x[t].v[i];
+            }
+    }
+    // the row's value on top of `base`: (base + sum1) + sum0 in MODE_DUAL, base + sum otherwise
+    __device__ __forceinline__ T total(T base, int t, int i) const {
+        if constexpr (MODE == MODE_DUAL) return (base + a[1][t].v[i]) + a[0][t].v[i];
+        else return base + a[0][t].v[i];
+    }
+};
 
 // Y[row] = (accumulate ? Y[row] : 0) + acc
-template <typename T, int VEC, int TILES>
+template <typename T, int VEC, int TILES, int MODE>
 __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_t foff[TILES],
-                                          const Pack<T, VEC> acc[TILES], int accumulate) {
+                                          const Acc<T, VEC, TILES, MODE> &acc, int accumulate) {
     T *yrow = Y + (int64_t)row * F;
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
@@ -100,42 +140,36 @@ __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_
             for (int i = 0; i < VEC; ++i) o.v[i] = T(0);
         }
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) o.v[i] = o.v[i] + acc[t].v[i];
+        for (int i = 0; i < VEC; ++i) o.v[i] = acc.total(o.v[i], t, i);
         store_pack<T, VEC>(yrow + foff[t], o);
     }
 }
 
-// Gather one feature tile of row c of X (masked by M in MODE_RELU_MASK).
+// Gather one feature tile of column c (source chosen by `src` in MODE_DUAL, masked by
+// M in MODE_RELU_MASK).
 template <typename T, int VEC, int MODE>
-__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int64_t foff) {
+__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int src, int64_t foff) {
     Pack<T, VEC> x;
     if (foff < 0) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) x.v[i] = T(0);
         return x;
     }
+    const T *base = a.X;
+    if constexpr (MODE == MODE_DUAL) {
+        if (src) {
+            base = a.X1;
+            c -= a.split;
+        }
+    }
     const int64_t off = (int64_t)c * a.F + foff;
-    x = load_pack<T, VEC>(a.X + off);
+    x = load_pack<T, VEC>(base + off);
     if constexpr (MODE == MODE_RELU_MASK) {
         Pack<T, VEC> m = load_pack<T, VEC>(a.M + off);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) x.v[i] = (m.v[i] <= T(0)) ? T(0) : x.v[i];
     }
     return x;
-}
-
-template <typename T, int VEC, int TILES, int MODE>
-__device__ __forceinline__ void accumulate_entry(Pack<T, VEC> acc[TILES],
-                                                 const Pack<T, VEC> x[TILES], T w) {
-#pragma unroll
-    for (int t = 0; t < TILES; ++t)
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            if constexpr (MODE == MODE_VAL)
-                acc[t].v[i] = acc[t].v[i] + x[t].v[i] * w;
-            else
-                acc[t].v[i] = acc[t].v[i] + x[t].v[i];
-        }
 }
 
 // ---------------------------------------------------------------- row schedule --
@@ -146,13 +180,13 @@ __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
     int row = blockIdx.x * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
     if (row >= a.rows) return;
-    int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
+    const int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
-    Pack<T, VEC> acc[TILES];
-    zero_acc<T, VEC, TILES>(acc);
+    Acc<T, VEC, TILES, MODE> acc;
+    acc.clear();
     if (e0 == e1) {
-        if (!a.accumulate) write_row<T, VEC, TILES>(a.Y, a.F, row, foff, acc, 0);
+        if (!a.accumulate) write_row<T, VEC, TILES, MODE>(a.Y, a.F, row, foff, acc, 0);
         return;
     }
     for (int e = e0; e < e1; e += kUnroll) {
@@ -161,71 +195,19 @@ __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
         Pack<T, VEC> x[kUnroll][TILES];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            int idx = min(e + u, e1 - 1);
+            const int idx = min(e + u, e1 - 1);
             c[u] = a.colidx[idx];
             w[u] = a.val ? a.val[idx] : T(1);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
-            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], foff[t]);
+            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
-            if (e + u < e1) accumulate_entry<T, VEC, TILES, MODE>(acc, x[u], w[u]);
+            if (e + u < e1) acc.add(x[u], w[u], c[u] >= a.split);
     }
-    write_row<T, VEC, TILES>(a.Y, a.F, row, foff, acc, a.accumulate);
-}
-
-// Two blocks over the same rows in one pass: Y[row] = (sum A0 row) + (sum A1 row).
-template <typename T>
-struct PairArgs {
-    SpmmArgs<T> a0, a1;
-};
-
-template <typename T, int VEC, int LPR, int TILES>
-__device__ __forceinline__ void row_sum(const SpmmArgs<T> &a, int row, const int64_t foff[TILES],
-                                        Pack<T, VEC> acc[TILES]) {
-    int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
-    for (int e = e0; e < e1; e += kUnroll) {
-        int c[kUnroll];
-        T w[kUnroll];
-        Pack<T, VEC> x[kUnroll][TILES];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            int idx = min(e + u, e1 - 1);
-            c[u] = a.colidx[idx];
-            w[u] = a.val ? a.val[idx] : T(1);
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE_VAL>(a, c[u], foff[t]);
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-            if (e + u < e1) accumulate_entry<T, VEC, TILES, MODE_VAL>(acc, x[u], w[u]);
-    }
-}
-
-template <typename T, int VEC, int LPR, int TILES>
-__global__ __launch_bounds__(kBlock) void spmm_pair_kernel(PairArgs<T> p) {
-    constexpr int GPB = kBlock / LPR;
-    const int lane = threadIdx.x % LPR;
-    int row = blockIdx.x * GPB + threadIdx.x / LPR;
-    if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
-    if (row >= p.a0.rows) return;
-    int64_t foff[TILES];
-    feature_offsets<VEC, LPR, TILES>(p.a0.F, lane, foff);
-    Pack<T, VEC> s0[TILES], s1[TILES];
-    zero_acc<T, VEC, TILES>(s0);
-    zero_acc<T, VEC, TILES>(s1);
-    row_sum<T, VEC, LPR, TILES>(p.a0, row, foff, s0);
-    row_sum<T, VEC, LPR, TILES>(p.a1, row, foff, s1);
-    // (0 + s0) + s1, the order of two successive accumulating calls.
-#pragma unroll
-    for (int t = 0; t < TILES; ++t)
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) s0[t].v[i] = (T(0) + s0[t].v[i]) + s1[t].v[i];
-    write_row<T, VEC, TILES>(p.a0.Y, p.a0.F, row, foff, s0, 0);
+    write_row<T, VEC, TILES, MODE>(a.Y, a.F, row, foff, acc, a.accumulate);
 }
 
 // ---------------------------------------------------------------- nnz schedule --
@@ -256,8 +238,8 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     }
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
-    Pack<T, VEC> acc[TILES];
-    zero_acc<T, VEC, TILES>(acc);
+    Acc<T, VEC, TILES, MODE> acc;
+    acc.clear();
     int cur = a.rowidx[e0];
     for (int e = e0; e < e1; e += kUnroll) {
         int r[kUnroll], c[kUnroll];
@@ -265,26 +247,26 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
         Pack<T, VEC> x[kUnroll][TILES];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            int idx = min(e + u, e1 - 1);
+            const int idx = min(e + u, e1 - 1);
             r[u] = a.rowidx[idx];
             c[u] = a.colidx[idx];
-            if constexpr (MODE == MODE_VAL) w[u] = a.val[idx];
+            if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
             else w[u] = T(1);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
-            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], foff[t]);
+            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             if (e + u < e1) {
                 if (r[u] != cur) {
                     // row `cur` ends inside this run: finish it here
-                    write_row<T, VEC, TILES>(a.Y, a.F, cur, foff, acc, a.accumulate);
-                    zero_acc<T, VEC, TILES>(acc);
+                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur, foff, acc, a.accumulate);
+                    acc.clear();
                     cur = r[u];
                 }
-                accumulate_entry<T, VEC, TILES, MODE>(acc, x[u], w[u]);
+                acc.add(x[u], w[u], c[u] >= a.split);
             }
         }
     }
@@ -293,9 +275,14 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
         T *crow = a.carry + (int64_t)seg * a.F;
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
-            if (foff[t] >= 0) store_pack<T, VEC>(crow + foff[t], acc[t]);
+            if (foff[t] >= 0) {
+                Pack<T, VEC> o;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) o.v[i] = acc.total(T(0), t, i);
+                store_pack<T, VEC>(crow + foff[t], o);
+            }
     } else {
-        write_row<T, VEC, TILES>(a.Y, a.F, cur, foff, acc, a.accumulate);
+        write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur, foff, acc, a.accumulate);
     }
     if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = continues ? cur : -1;
 }
@@ -312,30 +299,32 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
     if constexpr (LPR == kWave) item = __builtin_amdgcn_readfirstlane(item);
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
-    Pack<T, VEC> acc[TILES];
+    Acc<T, VEC, TILES, MODE_UNIT> acc;
     if (item < a.nseg) {
         const int r = a.carry_row[item];
         if (r >= 0 && (item == 0 || a.carry_row[item - 1] != r)) {
-            zero_acc<T, VEC, TILES>(acc);
+            acc.clear();
             int s = item;
             do {
                 const T *crow = a.carry + (int64_t)s * a.F;
+                Pack<T, VEC> cval[TILES];
 #pragma unroll
-                for (int t = 0; t < TILES; ++t)
-                    if (foff[t] >= 0) {
-                        Pack<T, VEC> cval = load_pack<T, VEC>(crow + foff[t]);
+                for (int t = 0; t < TILES; ++t) {
+                    if (foff[t] >= 0) cval[t] = load_pack<T, VEC>(crow + foff[t]);
+                    else
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) acc[t].v[i] = acc[t].v[i] + cval.v[i];
-                    }
+                        for (int i = 0; i < VEC; ++i) cval[t].v[i] = T(0);
+                }
+                acc.add(cval, T(1), 0);
                 ++s;
             } while (s < a.nseg && a.carry_row[s] == r);
-            write_row<T, VEC, TILES>(a.Y, a.F, r, foff, acc, 1);
+            write_row<T, VEC, TILES, MODE_UNIT>(a.Y, a.F, r, foff, acc, 1);
         }
     }
     if (!a.accumulate && item < a.rows) {
         if (a.rowptr[item] == a.rowptr[item + 1]) {
-            zero_acc<T, VEC, TILES>(acc);
-            write_row<T, VEC, TILES>(a.Y, a.F, item, foff, acc, 0);
+            acc.clear();
+            write_row<T, VEC, TILES, MODE_UNIT>(a.Y, a.F, item, foff, acc, 0);
         }
     }
 }
@@ -345,10 +334,18 @@ struct Shape {
     int vec, lpr, tiles, grid_y;
 };
 
+int env_int(const char *name) {
+    const char *s = std::getenv(name);
+    return s ? std::atoi(s) : 0;
+}
+
 // Lane layout for a feature width: the widest vector the width and the pointers'
 // alignment allow, then as many lanes as a row needs (power of two, 4..64).
+// CGNN_SPMM_VEC / CGNN_SPMM_LPR (environment, read once) override the choice where the
+// result is a layout that exists; they are for tuning experiments.
 template <typename T>
 Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, const void *p3) {
+    static const int force_vec = env_int("CGNN_SPMM_VEC"), force_lpr = env_int("CGNN_SPMM_LPR");
     auto aligned = [&](size_t bytes) {
         auto ok = [&](const void *p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0; };
         return ok(p0) && ok(p1) && ok(p2) && ok(p3);
@@ -358,11 +355,14 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
     if (sizeof(T) == 4) {
         if (F % 4 == 0 && aligned(16)) s.vec = 4;
         else if (F % 2 == 0 && aligned(8)) s.vec = 2;
+        if (force_vec == 2 && s.vec == 4) s.vec = 2;
+        if (force_vec == 1) s.vec = 1;
     }
     const int64_t slots = F / s.vec;
     int lpr = pow2_ceil(slots);
     if (lpr < 4) lpr = 4;
     if (lpr > 64) lpr = 64;
+    if (force_lpr >= 4 && force_lpr <= 64 && (force_lpr & (force_lpr - 1)) == 0 && force_lpr < lpr) lpr = force_lpr;
     if (s.vec != 4 || sizeof(T) != 4) {
         // fewer instantiations off the main path: 4, 16 or 64 lanes per row
         lpr = lpr <= 4 ? 4 : (lpr <= 16 ? 16 : 64);
@@ -373,45 +373,43 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
     return s;
 }
 
-enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2, KIND_PAIR = 3 };
+enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2 };
 
 template <typename T, int VEC, int LPR, int TILES>
-int launch_shape(int kind, int mode, const SpmmArgs<T> &a, const SpmmArgs<T> *a1, int64_t items,
-                 int grid_y, hipStream_t stream) {
+int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int grid_y, hipStream_t stream) {
     constexpr int GPB = kBlock / LPR;
     dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
     if (grid.x == 0) return CGNN_OK;
     switch (kind) {
         case KIND_ROW:
-            hipLaunchKernelGGL((spmm_row_kernel<T, VEC, LPR, TILES, MODE_VAL>), grid, block, 0, stream, a);
+            if (mode == MODE_DUAL)
+                hipLaunchKernelGGL((spmm_row_kernel<T, VEC, LPR, TILES, MODE_DUAL>), grid, block, 0, stream, a);
+            else
+                hipLaunchKernelGGL((spmm_row_kernel<T, VEC, LPR, TILES, MODE_VAL>), grid, block, 0, stream, a);
             break;
         case KIND_NNZ:
             if (mode == MODE_VAL)
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_VAL>), grid, block, 0, stream, a);
             else if (mode == MODE_UNIT)
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_UNIT>), grid, block, 0, stream, a);
+            else if (mode == MODE_DUAL)
+                hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_DUAL>), grid, block, 0, stream, a);
             else
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_RELU_MASK>), grid, block, 0, stream, a);
             break;
         case KIND_FIXUP:
             hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR, TILES>), grid, block, 0, stream, a);
             break;
-        case KIND_PAIR: {
-            PairArgs<T> p{a, *a1};
-            hipLaunchKernelGGL((spmm_pair_kernel<T, VEC, LPR, TILES>), grid, block, 0, stream, p);
-            break;
-        }
     }
     return check_launch("spmm launch");
 }
 
 #define CGNN_SHAPE_CASE(V, L, TL)                   \
     if (s.vec == V && s.lpr == L && s.tiles == TL)  \
-        return launch_shape<T, V, L, TL>(kind, mode, a, a1, items, s.grid_y, stream);
+        return launch_shape<T, V, L, TL>(kind, mode, a, items, s.grid_y, stream);
 
 template <typename T>
-int launch(int kind, int mode, const Shape &s, const SpmmArgs<T> &a, const SpmmArgs<T> *a1,
-           int64_t items, hipStream_t stream) {
+int launch(int kind, int mode, const Shape &s, const SpmmArgs<T> &a, int64_t items, hipStream_t stream) {
     if constexpr (sizeof(T) == 4) {
         CGNN_SHAPE_CASE(4, 4, 1)
         CGNN_SHAPE_CASE(4, 8, 1)
@@ -447,7 +445,8 @@ int resolve_kernel(const cgnn_csr *A, int kernel) {
 }
 
 int seg_len(const cgnn_csr *A) {
-    int s = A->seg_nnz > 0 ? A->seg_nnz : kDefaultSeg;
+    static const int force_seg = env_int("CGNN_SPMM_SEG");
+    int s = A->seg_nnz > 0 ? A->seg_nnz : (force_seg > 0 ? force_seg : kDefaultSeg);
     return (s + kUnroll - 1) / kUnroll * kUnroll;
 }
 
@@ -466,19 +465,21 @@ int check_csr(const cgnn_csr *A, const char *name) {
 }
 
 template <typename T>
-SpmmArgs<T> make_args(const cgnn_csr *A, const void *X, const void *M, void *Y, int64_t F,
-                      int accumulate) {
+SpmmArgs<T> make_args(const cgnn_csr *A, const void *X, const void *X1, int64_t split, const void *M, void *Y,
+                      int64_t F, int accumulate) {
     SpmmArgs<T> a{};
     a.rowptr = A->rowptr;
     a.colidx = A->colidx;
     a.rowidx = A->rowidx;
     a.val = static_cast<const T *>(A->val);
     a.X = static_cast<const T *>(X);
+    a.X1 = static_cast<const T *>(X1);
     a.M = static_cast<const T *>(M);
     a.Y = static_cast<T *>(Y);
     a.F = F;
     a.rows = (int32_t)A->rows;
     a.nnz = (int32_t)A->nnz;
+    a.split = (int32_t)split;
     a.accumulate = accumulate ? 1 : 0;
     return a;
 }
@@ -486,16 +487,19 @@ SpmmArgs<T> make_args(const cgnn_csr *A, const void *X, const void *M, void *Y, 
 size_t carry_row_bytes(int64_t nseg) { return align_up((size_t)nseg * sizeof(int32_t), 256); }
 
 template <typename T>
-int spmm_typed(const cgnn_csr *A, const void *X, const void *M, void *Y, int64_t F, int accumulate,
-               int kernel, int mode, void *ws, size_t ws_bytes, hipStream_t stream) {
+int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, const void *M, void *Y, int64_t F,
+               int accumulate, int kernel, int mode, void *ws, size_t ws_bytes, hipStream_t stream) {
     if (A->rows == 0 || F == 0) return CGNN_OK;
-    SpmmArgs<T> a = make_args<T>(A, X, M, Y, F, accumulate);
+    if (mode != MODE_DUAL) split = INT32_MAX;  // every column comes from X
+    SpmmArgs<T> a = make_args<T>(A, X, X1, split, M, Y, F, accumulate);
     kernel = resolve_kernel(A, kernel);
     if (mode == MODE_RELU_MASK) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
     if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;
+    if (mode == MODE_DUAL && A->nnz > 0 && A->val == nullptr)
+        return fail(CGNN_EINVAL, "spmm: the two-source product needs stored values");
     if (kernel == CGNN_SPMM_ROW) {
-        Shape s = pick_shape<T>(F, X, Y, nullptr, nullptr);
-        return launch<T>(KIND_ROW, mode, s, a, nullptr, A->rows, stream);
+        Shape s = pick_shape<T>(F, X, Y, X1, nullptr);
+        return launch<T>(KIND_ROW, mode, s, a, A->rows, stream);
     }
     if (A->nnz > 0 && A->rowidx == nullptr) return fail(CGNN_EINVAL, "spmm: nnz schedule needs rowidx");
     const int seg = seg_len(A);
@@ -509,89 +513,16 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *M, void *Y, int64_t
     a.seg_nnz = seg;
     a.carry_row = static_cast<int32_t *>(ws);
     a.carry = reinterpret_cast<T *>(static_cast<char *>(ws) + carry_row_bytes(nseg));
-    Shape s = pick_shape<T>(F, X, Y, a.carry, M);
+    Shape s = pick_shape<T>(F, X, Y, nseg > 0 ? a.carry : nullptr, mode == MODE_DUAL ? X1 : M);
     if (nseg > 0) {
-        int rc = launch<T>(KIND_NNZ, mode, s, a, nullptr, nseg, stream);
+        int rc = launch<T>(KIND_NNZ, mode, s, a, nseg, stream);
         if (rc != CGNN_OK) return rc;
     }
     const int64_t items = accumulate ? nseg : (nseg > A->rows ? nseg : A->rows);
-    return launch<T>(KIND_FIXUP, mode, s, a, nullptr, items, stream);
-}
-
-}  // namespace
-
-// Entry used by the cluster reductions (unit values, optional ReLU mask).
-int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, void *Y, int64_t F,
-                 bool relu_mask, void *ws, size_t ws_bytes, hipStream_t stream) {
-    const int mode = relu_mask ? MODE_RELU_MASK : MODE_UNIT;
-    if (dtype == CGNN_F32)
-        return spmm_typed<float>(A, X, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
-    if (dtype == CGNN_F64)
-        return spmm_typed<double>(A, X, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
-    return fail(CGNN_EUNSUPPORTED, "spmm: dtype must be f32 or f64");
-}
-
-}  // namespace cgnn
-
-using namespace cgnn;
-
-extern "C" size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dtype, int kernel) {
-    if (A == nullptr || A->nnz <= 0 || F <= 0) return 0;
-    if (resolve_kernel(A, kernel) == CGNN_SPMM_ROW) return 0;
-    const int64_t nseg = ceil_div(A->nnz, seg_len(A));
-    const size_t elt = dtype == CGNN_F64 ? 8 : 4;
-    return carry_row_bytes(nseg) + (size_t)nseg * (size_t)F * elt;
-}
-
-extern "C" int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
-                         int accumulate, int kernel, void *workspace, size_t workspace_bytes,
-                         cgnn_stream_t stream) {
-    int rc = check_csr(A, "cgnn_spmm");
-    if (rc != CGNN_OK) return rc;
-    CGNN_REQUIRE(F >= 0, "cgnn_spmm: F must be non-negative");
-    if (A->rows == 0 || F == 0) return CGNN_OK;
-    CGNN_REQUIRE(Y != nullptr, "cgnn_spmm: Y is null");
-    CGNN_REQUIRE(A->nnz == 0 || X != nullptr, "cgnn_spmm: X is null");
-    CGNN_REQUIRE(kernel >= CGNN_SPMM_AUTO && kernel <= CGNN_SPMM_NNZ, "cgnn_spmm: unknown kernel id");
-    if (dtype == CGNN_F32)
-        return spmm_typed<float>(A, X, nullptr, Y, F, accumulate, kernel, MODE_VAL, workspace,
-                                 workspace_bytes, stream);
-    if (dtype == CGNN_F64)
-        return spmm_typed<double>(A, X, nullptr, Y, F, accumulate, kernel, MODE_VAL, workspace,
-                                  workspace_bytes, stream);
-    return fail(CGNN_EUNSUPPORTED, "cgnn_spmm: dtype must be f32 or f64");
-}
-
-template <typename T>
-static int spmm_pair_typed(const cgnn_csr *A0, const void *X0, const cgnn_csr *A1, const void *X1,
-                           void *Y, int64_t F, hipStream_t stream) {
-    SpmmArgs<T> a0 = make_args<T>(A0, X0, nullptr, Y, F, 0);
-    SpmmArgs<T> a1 = make_args<T>(A1, X1, nullptr, Y, F, 0);
-    Shape s = pick_shape<T>(F, X0, X1, Y, nullptr);
-    return launch<T>(KIND_PAIR, MODE_VAL, s, a0, &a1, A0->rows, stream);
-}
-
-extern "C" int cgnn_spmm_pair(const cgnn_csr *A0, const void *X0, const cgnn_csr *A1,
-                              const void *X1, int dtype, void *Y, int64_t F,
-                              cgnn_stream_t stream) {
-    int rc = check_csr(A0, "cgnn_spmm_pair(A0)");
-    if (rc != CGNN_OK) return rc;
-    rc = check_csr(A1, "cgnn_spmm_pair(A1)");
-    if (rc != CGNN_OK) return rc;
-    CGNN_REQUIRE(A0->rows == A1->rows, "cgnn_spmm_pair: blocks must have the same number of rows");
-    CGNN_REQUIRE(F >= 0, "cgnn_spmm_pair: F must be non-negative");
-    if (A0->rows == 0 || F == 0) return CGNN_OK;
-    CGNN_REQUIRE(Y != nullptr, "cgnn_spmm_pair: Y is null");
-    CGNN_REQUIRE((A0->nnz == 0 || X0 != nullptr) && (A1->nnz == 0 || X1 != nullptr),
-                 "cgnn_spmm_pair: X is null");
-    if (dtype == CGNN_F32) return spmm_pair_typed<float>(A0, X0, A1, X1, Y, F, stream);
-    if (dtype == CGNN_F64) return spmm_pair_typed<double>(A0, X0, A1, X1, Y, F, stream);
-    return fail(CGNN_EUNSUPPORTED, "cgnn_spmm_pair: dtype must be f32 or f64");
+    return launch<T>(KIND_FIXUP, mode, s, a, items, stream);
 }
 
 // ------------------------------------------------------- CSR preparation -------
-namespace cgnn {
-namespace {
 
 __global__ void narrow_i64_kernel(const int64_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
@@ -621,7 +552,69 @@ unsigned grid_for(int64_t n) {
 }
 
 }  // namespace
+
+// Entry used by the cluster reductions (unit values, optional ReLU mask).
+int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, void *Y, int64_t F,
+                 bool relu_mask, void *ws, size_t ws_bytes, hipStream_t stream) {
+    const int mode = relu_mask ? MODE_RELU_MASK : MODE_UNIT;
+    if (dtype == CGNN_F32)
+        return spmm_typed<float>(A, X, nullptr, 0, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
+    if (dtype == CGNN_F64)
+        return spmm_typed<double>(A, X, nullptr, 0, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
+    return fail(CGNN_EUNSUPPORTED, "spmm: dtype must be f32 or f64");
+}
+
 }  // namespace cgnn
+
+using namespace cgnn;
+
+extern "C" size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dtype, int kernel) {
+    if (A == nullptr || A->nnz <= 0 || F <= 0) return 0;
+    if (resolve_kernel(A, kernel) == CGNN_SPMM_ROW) return 0;
+    const int64_t nseg = ceil_div(A->nnz, seg_len(A));
+    const size_t elt = dtype == CGNN_F64 ? 8 : 4;
+    return carry_row_bytes(nseg) + (size_t)nseg * (size_t)F * elt;
+}
+
+extern "C" int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
+                         int accumulate, int kernel, void *workspace, size_t workspace_bytes,
+                         cgnn_stream_t stream) {
+    int rc = check_csr(A, "cgnn_spmm");
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(F >= 0, "cgnn_spmm: F must be non-negative");
+    if (A->rows == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(Y != nullptr, "cgnn_spmm: Y is null");
+    CGNN_REQUIRE(A->nnz == 0 || X != nullptr, "cgnn_spmm: X is null");
+    CGNN_REQUIRE(kernel >= CGNN_SPMM_AUTO && kernel <= CGNN_SPMM_NNZ, "cgnn_spmm: unknown kernel id");
+    if (dtype == CGNN_F32)
+        return spmm_typed<float>(A, X, nullptr, 0, nullptr, Y, F, accumulate, kernel, MODE_VAL, workspace,
+                                 workspace_bytes, stream);
+    if (dtype == CGNN_F64)
+        return spmm_typed<double>(A, X, nullptr, 0, nullptr, Y, F, accumulate, kernel, MODE_VAL, workspace,
+                                  workspace_bytes, stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_spmm: dtype must be f32 or f64");
+}
+
+extern "C" int cgnn_spmm_dual(const cgnn_csr *A, int64_t split, int dtype, const void *X0, const void *X1,
+                              void *Y, int64_t F, int kernel, void *workspace, size_t workspace_bytes,
+                              cgnn_stream_t stream) {
+    int rc = check_csr(A, "cgnn_spmm_dual");
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(F >= 0, "cgnn_spmm_dual: F must be non-negative");
+    CGNN_REQUIRE(split >= 0 && split <= A->cols, "cgnn_spmm_dual: split must be in [0, cols]");
+    if (A->rows == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(Y != nullptr, "cgnn_spmm_dual: Y is null");
+    CGNN_REQUIRE(A->nnz == 0 || ((split == 0 || X0 != nullptr) && (split == A->cols || X1 != nullptr)),
+                 "cgnn_spmm_dual: a source matrix is null");
+    CGNN_REQUIRE(kernel >= CGNN_SPMM_AUTO && kernel <= CGNN_SPMM_NNZ, "cgnn_spmm_dual: unknown kernel id");
+    if (dtype == CGNN_F32)
+        return spmm_typed<float>(A, X0, X1, split, nullptr, Y, F, 0, kernel, MODE_DUAL, workspace, workspace_bytes,
+                                 stream);
+    if (dtype == CGNN_F64)
+        return spmm_typed<double>(A, X0, X1, split, nullptr, Y, F, 0, kernel, MODE_DUAL, workspace, workspace_bytes,
+                                  stream);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_spmm_dual: dtype must be f32 or f64");
+}
 
 extern "C" int cgnn_csr_prepare_i64(int64_t rows, int64_t nnz, const int64_t *rowptr64,
                                     const int64_t *col64, int32_t *rowptr32, int32_t *col32,

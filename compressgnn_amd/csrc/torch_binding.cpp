@@ -245,8 +245,10 @@ struct StageTimer {
 struct PropagationPlan {
     std::shared_ptr<DeviceCsr> v2v, v2r, r2v, v2v_t, v2r_t, r2v_t;
     std::vector<std::shared_ptr<DeviceCsr>> r2r, r2r_t;
+    // [v2v | v2r] and [v2v^T | r2v^T]: the vertex stage of forward / backward in one pass
+    std::shared_ptr<DeviceCsr> vertex_stage, vertex_stage_t;
     int64_t V = 0, R = 0;
-    bool fuse_final = true;  // last two stages in one pass (cgnn_spmm_pair)
+    bool fuse_final = true;  // last two stages in one pass (cgnn_spmm_dual)
     int kernel = CGNN_SPMM_AUTO;
     StageTimer timer;
 };
@@ -260,18 +262,21 @@ Tensor timed_spmm(PropagationPlan &p, const std::string &stage, DeviceCsr &A, co
     return r;
 }
 
-Tensor final_stage(PropagationPlan &p, const std::string &prefix, DeviceCsr &from_rules, const Tensor &rule_x,
-                   DeviceCsr &from_vertices, const Tensor &x) {
+Tensor final_stage(PropagationPlan &p, const std::string &prefix, DeviceCsr *merged, DeviceCsr &from_rules,
+                   const Tensor &rule_x, DeviceCsr &from_vertices, const Tensor &x) {
     const int64_t F = x.size(1);
-    if (p.fuse_final) {
-        Tensor out = torch::empty({from_vertices.rows, F}, x.options());
+    if (p.fuse_final && merged != nullptr) {
+        Tensor out = torch::empty({merged->rows, F}, x.options());
         if (out.numel() == 0) return out;
+        const int dtype = dtype_code(x);
+        size_t bytes = 0;
+        Tensor ws = merged->workspace(F, dtype, p.kernel, &bytes);
         hipStream_t stream = reinterpret_cast<hipStream_t>(current_stream(x));
         const int id = p.timer.open(prefix + "final", stream);
-        cgnn_csr a0 = from_rules.view(), a1 = from_vertices.view();
-        ok(cgnn_spmm_pair(&a0, rule_x.data_ptr(), &a1, x.data_ptr(), dtype_code(x), out.data_ptr(), F,
-                          current_stream(x)),
-           "spmm_pair");
+        cgnn_csr a = merged->view();
+        ok(cgnn_spmm_dual(&a, from_vertices.cols, dtype, x.data_ptr(), rule_x.data_ptr(), out.data_ptr(), F, p.kernel,
+                          ws.data_ptr(), bytes, current_stream(x)),
+           "spmm_dual");
         p.timer.close(id, stream);
         return out;
     }
@@ -289,7 +294,7 @@ Tensor propagate_forward(PropagationPlan &p, Tensor x) {
     Tensor rule_out = timed_spmm(p, "fwd.rules", *p.r2v, x, c10::nullopt);
     for (size_t i = 0; i < p.r2r.size(); ++i)
         rule_out = timed_spmm(p, "fwd.level" + std::to_string(i), *p.r2r[i], rule_out, rule_out);
-    return final_stage(p, "fwd.", *p.v2r, rule_out, *p.v2v, x);
+    return final_stage(p, "fwd.", p.vertex_stage.get(), *p.v2r, rule_out, *p.v2v, x);
 }
 
 // layer/CompressgnnSPMM.py:65-86 (the working branch, lines 80-85).  Stage names as in
@@ -302,7 +307,7 @@ Tensor propagate_backward(PropagationPlan &p, Tensor grad) {
     Tensor rule_g = timed_spmm(p, "bwd.rules", *p.v2r_t, grad, c10::nullopt);
     for (size_t i = p.r2r_t.size(); i-- > 0;)
         rule_g = timed_spmm(p, "bwd.level" + std::to_string(i), *p.r2r_t[i], rule_g, rule_g);
-    return final_stage(p, "bwd.", *p.r2v_t, rule_g, *p.v2v_t, grad);
+    return final_stage(p, "bwd.", p.vertex_stage_t.get(), *p.r2v_t, rule_g, *p.v2v_t, grad);
 }
 
 // ---------------------------------------------------- transformation compression ----
@@ -560,6 +565,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
                  return p;
              }))
         .def_readwrite("fuse_final", &PropagationPlan::fuse_final)
+        .def_readwrite("vertex_stage", &PropagationPlan::vertex_stage)
+        .def_readwrite("vertex_stage_t", &PropagationPlan::vertex_stage_t)
         .def_property("method",
                       [](PropagationPlan &p) { return p.kernel == CGNN_SPMM_ROW ? "rowbalance" : p.kernel == CGNN_SPMM_NNZ ? "nnzbalance" : "auto"; },
                       [](PropagationPlan &p, std::string mth) { p.kernel = kernel_of_method(mth); })

@@ -6,7 +6,7 @@ loader/compress_graph.py:6-57; on a GPU it additionally carries the propagation 
 import _paths  # noqa: F401
 import torch
 
-from compressgnn_offline import gen_degree, hybird_partition, topo_partition
+from compressgnn_offline import csr_hstack, gen_degree, hybird_partition, topo_partition
 from sparse_csr import SparseCSR
 
 
@@ -72,7 +72,16 @@ class CompressGraph():
                 cp, row, val = g.csc()
                 return rt.DeviceCsr(cp, row, val, g.sparse_size(1), g.sparse_size(0), dev)
 
-            self._plan = rt.PropagationPlan(
+            plan = rt.PropagationPlan(
                 fwd(self.v2v_graph), fwd(self.v2r_graph), fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
                 bwd(self.v2v_graph), bwd(self.v2r_graph), bwd(self.r2v_graph), [bwd(g) for g in self.r2r_graph])
+            # the vertex stage reads [v2v | v2r] (forward) and [v2v^T | r2v^T] (backward) in one pass
+            V, R = self.vertex_cnt, self.rule_cnt
+            host = lambda triple: tuple(t.cpu().numpy() for t in triple)
+            t = torch.from_numpy
+            rp, ci, val = csr_hstack(host(self.v2v_graph.csr()), host(self.v2r_graph.csr()), V)
+            plan.vertex_stage = rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev)
+            rp, ci, val = csr_hstack(host(self.v2v_graph.csc()), host(self.r2v_graph.csc()), V)
+            plan.vertex_stage_t = rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev)
+            self._plan = plan
         return self._plan

@@ -82,14 +82,17 @@ int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
               int accumulate, int kernel, void *workspace, size_t workspace_bytes,
               cgnn_stream_t stream);
 
-/* Y[rows x F] = A0 * X0 + A1 * X1 in one pass over the rows (A0 and A1 have the same
- * number of rows).  Each row is summed as (sum over A0's entries) + (sum over A1's
- * entries), which is the value the two-call sequence
+/* Two-source product in one pass: A has `cols` columns; a column c < split gathers
+ * row c of X0, a column c >= split gathers row c - split of X1.  Every row of Y is
+ * written as (0 + S1) + S0 with S1 / S0 the sums over the row's X1 / X0 entries, each
+ * in storage order -- the value the two-call sequence
  *   out = spmm(v2r, rule_out, None); out = spmm(v2v, x, out)
- * of layer/CompressgnnSPMM.py:59-60 (and 84-85 in backward) produces, without
- * reading Y back.  ROW schedule only (A0/A1 rowidx unused). */
-int cgnn_spmm_pair(const cgnn_csr *A0, const void *X0, const cgnn_csr *A1, const void *X1,
-                   int dtype, void *Y, int64_t F, cgnn_stream_t stream);
+ * of layer/CompressgnnSPMM.py:59-60 (84-85 in backward) produces when A's rows are
+ * [v2v row | v2r row with columns shifted by split = vertex_cnt], without writing Y
+ * twice or reading it back.  A->val must not be NULL.  Workspace as for cgnn_spmm. */
+int cgnn_spmm_dual(const cgnn_csr *A, int64_t split, int dtype, const void *X0, const void *X1,
+                   void *Y, int64_t F, int kernel, void *workspace, size_t workspace_bytes,
+                   cgnn_stream_t stream);
 
 /* Widen-free preparation of a CSR given as int64 tensors (the layout
  * src/runtime/csrc/sparse/cuda/spmm_gpu.cu:38-46 reads): converts rowptr/col to

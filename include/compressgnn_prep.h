@@ -94,6 +94,13 @@ cgnn_arrays *cgnn_gen_vertex_order_csc(int64_t V, int64_t R, const int64_t *vlis
 cgnn_arrays *cgnn_compress_csr_batch(int64_t V, const int64_t *vlist, const int64_t *elist,
                                      int threads, int rounds, int min_pair_frequency);
 
+/* [A0 | A1]: row r of the result is row r of A0 followed by row r of A1 with its
+ * columns shifted by col_offset (the vertex stage of the propagation reads the
+ * vertex->vertex and vertex->rule blocks this way in one pass). -> [vlist, elist, value] */
+cgnn_arrays *cgnn_csr_hstack(int64_t rows, const int64_t *vlist0, const int64_t *elist0, const float *value0,
+                             const int64_t *vlist1, const int64_t *elist1, const float *value1,
+                             int64_t col_offset);
+
 /* Longest row, and a histogram of row lengths in powers of two:
  * hist[k] = rows with length in [2^(k-1), 2^k) for k >= 1, hist[0] = empty rows. */
 int cgnn_csr_row_stats(int64_t rows, const int64_t *vlist, int64_t *max_row, int64_t hist[40]);

@@ -116,20 +116,37 @@ def test_spmm_in_place_levels():
         assert np.array_equal(Z.cpu().numpy(), want)
 
 
-def test_spmm_pair_equals_two_calls():
-    rng = np.random.default_rng(13)
-    V, R, F = 500, 120, 128
-    a0 = random_csr(rng, V, R, 2.0)
-    a1 = random_csr(rng, V, V, 7.0)
+@pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
+@pytest.mark.parametrize("F", [16, 128, 130])
+def test_spmm_dual_equals_two_calls(kernel, F):
+    """[A1 | A0] in one pass == spmm(A0, x_rules) then spmm(A1, x_vertices, out=...),
+    bit for bit on rows that fit in one run."""
+    rng = np.random.default_rng(13 + F)
+    V, R = 500, 120
+    a0 = random_csr(rng, V, R, 2.0)              # vertex <- rule entries
+    a1 = random_csr(rng, V, V, 7.0, skew=True)   # vertex <- vertex entries
+    scale = lambda a: (a[0], a[1], (a[2] * 0.05).astype(np.float32))
+    a0, a1 = scale(a0), scale(a1)
     xr = rng.standard_normal((R, F)).astype(np.float32)
     xv = rng.standard_normal((V, F)).astype(np.float32)
     want = oracle.spmm(*a0, xr)
     want = oracle.spmm(*a1, xv, want)
-    A0 = abi.DeviceCsr.from_host(V, R, *a0, DEV)
-    A1 = abi.DeviceCsr.from_host(V, V, *a1, DEV)
-    got = abi.spmm_pair(A0, torch.from_numpy(xr).to(DEV), A1, torch.from_numpy(xv).to(DEV))
+    # merged rows: vertex columns first, then rule columns shifted by V
+    ptr = a1[0] + a0[0]
+    col = np.concatenate([np.concatenate([a1[1][a1[0][r]:a1[0][r + 1]], a0[1][a0[0][r]:a0[0][r + 1]] + V])
+                          for r in range(V)]).astype(np.int64)
+    val = np.concatenate([np.concatenate([a1[2][a1[0][r]:a1[0][r + 1]], a0[2][a0[0][r]:a0[0][r + 1]]])
+                          for r in range(V)]).astype(np.float32)
+    A = abi.DeviceCsr.from_host(V, V + R, ptr, col, val, DEV)
+    got = abi.spmm_dual(A, V, torch.from_numpy(xv).to(DEV), torch.from_numpy(xr).to(DEV), None, kernel)
     torch.cuda.synchronize()
-    assert np.array_equal(got.cpu().numpy(), want)
+    got = got.cpu().numpy()
+    assert_within(got, want)
+    short = np.diff(ptr) <= 64
+    if kernel == abi.SPMM_ROW:
+        assert np.array_equal(got, want)
+    else:
+        assert np.array_equal(got[short], want[short])
 
 
 def test_spmm_f64():
