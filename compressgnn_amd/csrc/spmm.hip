@@ -73,6 +73,19 @@ template <typename T, int VEC>
 __device__ __forceinline__ void store_pack(T *p, const Pack<T, VEC> &x) {
     *reinterpret_cast<Pack<T, VEC> *>(p) = x;
 }
+// Streaming store for rows that are written once and not read again by this launch.
+template <typename T, int VEC>
+__device__ __forceinline__ void store_pack_stream(T *p, const Pack<T, VEC> &x) {
+    if constexpr (VEC == 1) {
+        __builtin_nontemporal_store(x.v[0], p);
+    } else {
+        typedef T vec_t __attribute__((ext_vector_type(VEC)));
+        vec_t v;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = x.v[i];
+        __builtin_nontemporal_store(v, reinterpret_cast<vec_t *>(p));
+    }
+}
 
 // Per-lane feature offsets of the TILES tiles; foff[t] < 0 marks a tile beyond F.
 template <int VEC, int LPR, int TILES>
@@ -84,43 +97,52 @@ __device__ __forceinline__ void feature_offsets(int64_t F, int lane, int64_t fof
     }
 }
 
-// Accumulators of one output row: one set, or two in MODE_DUAL.
+// Accumulators of one output row: one set, or two in MODE_DUAL (separate members, so
+// that both stay in registers).
 template <typename T, int VEC, int TILES, int MODE>
 struct Acc {
-    static constexpr int SETS = MODE == MODE_DUAL ? 2 : 1;
-    Pack<T, VEC> a[SETS][TILES];
+    Pack<T, VEC> a0[TILES];
+    Pack<T, VEC> a1[MODE == MODE_DUAL ? TILES : 1];
 
     __device__ __forceinline__ void clear() {
-#pragma unroll
-        for (int s = 0; s < SETS; ++s)
-#pragma unroll
-            for (int t = 0; t < TILES; ++t)
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) a[s][t].v[i] = T(0);
-    }
-    // entry with gathered tiles x, value w, from source `src` (0 or 1)
-    __device__ __forceinline__ void add(const Pack<T, VEC> x[TILES], T w, int src) {
-        if constexpr (MODE == MODE_DUAL) {
-            if (src) {
-#pragma unroll
-                for (int t = 0; t < TILES; ++t)
-#pragma unroll
-                    for (int i = 0; i < VEC; ++i) a[1][t].v[i] = a[1][t].v[i] + x[t].v[i] * w;
-                return;
-            }
-        }
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) a[0][t].v[i] = a[0][t].v[i] + x[t].v[i] * w;
-                else a[0][t].v[i] = a[0][t].v[i] + x[t].v[i];
+                a0[t].v[i] = T(0);
+                if constexpr (MODE == MODE_DUAL) a1[t].v[i] = T(0);
             }
+    }
+    // entry with gathered tiles x, value w, from source `src` (0 or 1)
+    __device__ __forceinline__ void add(const Pack<T, VEC> x[TILES], T w, int src) {
+        if constexpr (MODE == MODE_DUAL) {
+            // Both updates are formed and one is kept by a value select.  A branch on
+            // `src` would be turned into an indexed access to the two accumulator sets,
+            // which moves them out of registers into scratch memory.
+            const bool second = src != 0;
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const T p = x[t].v[i] * w;
+                    const T u0 = a0[t].v[i] + p, u1 = a1[t].v[i] + p;
+                    a0[t].v[i] = second ? a0[t].v[i] : u0;
+                    a1[t].v[i] = second ? u1 : a1[t].v[i];
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    if constexpr (MODE == MODE_VAL) a0[t].v[i] = a0[t].v[i] + x[t].v[i] * w;
+                    else a0[t].v[i] = a0[t].v[i] + x[t].v[i];
+                }
+        }
     }
     // the row's value on top of `base`: (base + sum1) + sum0 in MODE_DUAL, base + sum otherwise
     __device__ __forceinline__ T total(T base, int t, int i) const {
-        if constexpr (MODE == MODE_DUAL) return (base + a[1][t].v[i]) + a[0][t].v[i];
-        else return base + a[0][t].v[i];
+        if constexpr (MODE == MODE_DUAL) return (base + a1[t].v[i]) + a0[t].v[i];
+        else return base + a0[t].v[i];
     }
 };
 
@@ -141,7 +163,8 @@ __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) o.v[i] = acc.total(o.v[i], t, i);
-        store_pack<T, VEC>(yrow + foff[t], o);
+        if (accumulate) store_pack<T, VEC>(yrow + foff[t], o);
+        else store_pack_stream<T, VEC>(yrow + foff[t], o);
     }
 }
 

@@ -125,7 +125,7 @@ def test_spmm_dual_equals_two_calls(kernel, F):
     V, R = 500, 120
     a0 = random_csr(rng, V, R, 2.0)              # vertex <- rule entries
     a1 = random_csr(rng, V, V, 7.0, skew=True)   # vertex <- vertex entries
-    scale = lambda a: (a[0], a[1], (a[2] * 0.05).astype(np.float32))
+    scale = lambda a: (a[0], a[1], (a[2] * 0.3 / np.sqrt(np.maximum(np.repeat(np.diff(a[0]), np.diff(a[0])), 1))).astype(np.float32))
     a0, a1 = scale(a0), scale(a1)
     xr = rng.standard_normal((R, F)).astype(np.float32)
     xv = rng.standard_normal((V, F)).astype(np.float32)
