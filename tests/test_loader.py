@@ -1,0 +1,125 @@
+"""CompressgnnData / CompressGraph on the host: fields and repr of the reference's
+loader, block shapes, the expansion invariant (the blocks reproduce the original graph
+with self loops), weights along every expanded path, and level ordering."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path[:0] = [os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compressgnn_amd", "layer"),
+                os.path.join(ROOT, "compressgnn_amd", "loader")]
+
+import compressgnn_offline as off  # noqa: E402
+from CompressgnnData import CompressgnnData  # noqa: E402
+from compress_graph import CompressGraph  # noqa: E402
+from sparse_csr import SparseCSR  # noqa: E402
+
+
+def make(kind, normalize=True, freq=3, add_self_loop=True):
+    if kind == "blocks":
+        n = 64
+        v = np.arange(n + 1, dtype=np.int32) * 32
+        e = np.tile(np.arange(32, dtype=np.int32), n)
+    else:
+        v, e = off.gen_copy_model(1500, 9.0, 0.7, 3)
+    V = len(v) - 1
+    x = np.random.default_rng(0).standard_normal((V, 8))
+    mask = np.ones(V, dtype=bool)
+    data = CompressgnnData(x, (v, e), np.zeros(V, np.int64), mask, mask, mask, add_self_loop=add_self_loop,
+                           normalize=normalize, graph_type="csr", min_pair_frequency=freq)
+    return data, np.asarray(v, np.int64), np.asarray(e, np.int64)
+
+
+def dense_of(graph, V, R):
+    """(V+R)-square matrix M with M[child, parent] = weight, from the blocks."""
+    M = np.zeros((V + R, V + R))
+    def put(g, r0, c0):
+        rp, ci, val = (t.numpy() for t in g.csr())
+        for r in range(len(rp) - 1):
+            for k in range(rp[r], rp[r + 1]):
+                M[r0 + r, c0 + ci[k]] += val[k]
+    put(graph.v2v_graph, 0, 0)
+    put(graph.v2r_graph, 0, V)
+    put(graph.r2v_graph, V, 0)
+    for g in graph.r2r_graph:
+        put(g, V, V)
+    return M
+
+
+@pytest.mark.parametrize("kind", ["blocks", "copy"])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_blocks_expand_to_the_original_graph(kind, normalize):
+    data, v, e = make(kind, normalize)
+    g = data.edge_index
+    V, R = data.vertex_cnt, data.rule_cnt
+    assert isinstance(g, CompressGraph) and R > 0
+    assert data.x.dtype == torch.float32 and data.feature_dim == 8 and data.graph_type == "csr"
+    assert repr(data).startswith('CompressgnnData(vertex_cnt:"%d", rule_cnt:"%d"' % (V, R)) and repr(g) == 'CompressGraph'
+    assert g.v2v_graph.sparse_sizes() == (V, V) and g.v2r_graph.sparse_sizes() == (V, R)
+    assert g.r2v_graph.sparse_sizes() == (R, V) and all(l.sparse_sizes() == (R, R) for l in g.r2r_graph)
+    assert g.step == len(g.r2r_graph)
+    for t in g.v2v_graph.csr()[:2]:
+        assert t.dtype == torch.int64
+    assert g.v2v_graph.csr()[2].dtype == torch.float32
+    # out = (I - N)^-1 restricted to vertices: propagate the identity through the blocks
+    M = dense_of(g, V, R)
+    vv, vr, rv, rr = M[:V, :V], M[:V, V:], M[V:, :V], M[V:, V:]
+    closure = np.linalg.inv(np.eye(R) - rr)  # rule levels are acyclic, so this is a finite sum
+    A_t = vv + vr @ closure @ rv             # A_hat^T as the compressed chain computes it
+    sv, se = off.add_self_loop_csr(v, e)
+    src = np.repeat(np.arange(V), np.diff(sv))
+    want = np.zeros((V, V))
+    if normalize:
+        d = off.get_norm_degree(se, V).astype(np.float64)
+        np.add.at(want, (se, src), d[src] * d[se])
+    else:
+        np.add.at(want, (se, src), 1.0)
+    np.testing.assert_allclose(A_t, want, rtol=1e-5, atol=1e-7)
+    # expanded degrees count the expanded in-edges
+    indeg = np.bincount(se, minlength=V)
+    assert np.array_equal(g.vertex_degree.numpy(), indeg)
+
+
+def test_csc_is_the_stable_transpose():
+    rng = np.random.default_rng(1)
+    rp = np.array([0, 3, 3, 6, 8])
+    ci = np.array([2, 0, 2, 1, 1, 0, 3, 2])  # duplicates inside rows keep their order
+    val = rng.standard_normal(8).astype(np.float32)
+    g = SparseCSR(rp, ci, val, (4, 4))
+    cp, row, tv = g.csc()
+    assert cp.tolist() == [0, 2, 4, 7, 8]
+    assert row.tolist() == [0, 2, 2, 2, 0, 0, 3, 3]
+    assert np.array_equal(tv.numpy(), val[[1, 5, 3, 4, 0, 2, 7, 6]])
+    assert g.t().sparse_sizes() == (4, 4) and g.to("cpu").nnz() == 8
+
+
+def test_unsupported_paths_fail_loudly():
+    with pytest.raises(NotImplementedError):
+        CompressgnnData(np.zeros((2, 1)), (np.array([0, 1]), np.array([1, 0])), np.zeros(2), np.ones(2, bool),
+                        np.ones(2, bool), np.ones(2, bool), graph_type="coo")
+    with pytest.raises(ValueError):
+        CompressgnnData(np.zeros((2, 1)), (np.array([0, 1, 2]), np.array([1, 0])), np.zeros(2), np.ones(2, bool),
+                        np.ones(2, bool), np.ones(2, bool), graph_type="csr", compression_backend="tpu")
+    data, _, _ = make("blocks")
+    from KPropagate import KPropagate
+    with pytest.raises(RuntimeError, match="GPU"):
+        KPropagate()(data.x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    with pytest.raises(RuntimeError, match="GPU"):
+        data.edge_index.plan()
+
+
+def test_backend_resolution():
+    import compression_backend as dispatch
+    assert dispatch.resolve_backend('auto') == 'cpu' and dispatch.resolve_backend('cpu') == 'cpu'
+    with pytest.raises(RuntimeError):
+        dispatch.resolve_backend('cuda')
+    for bad in ['wrong', 'legacy', None]:
+        with pytest.raises(ValueError):
+            dispatch.resolve_backend(bad)
+    with pytest.raises(ValueError):
+        dispatch.compress_graph_csr(np.array([0, 0]), np.array([], np.int64), 2)
+    with pytest.raises(ValueError):
+        dispatch.compress_graph_csr(np.array([0, 0]), np.array([], np.int64), 16, threads=0)
