@@ -219,11 +219,11 @@ def bench_cluster(torch, steps, detail):
     t_members, members = timed(lambda: rt.cluster_members(ids, groups))
     t_mean, reps = timed(lambda: rt.cluster_mean(x, ids, counts, members))
     t_linear, hidden = timed(lambda: torch.nn.functional.linear(reps, weight))
-    t_recon, out = timed(lambda: rt.cluster_reconstruct(hidden, ids, bias, True))
+    t_recon, out = timed(lambda: rt.cluster_reconstruct(hidden, ids, bias, True, members))
     grad_out = torch.randn(N, Fo, device=dev, generator=gen)
     t_recon_bwd, hidden_grad = timed(lambda: rt.cluster_reconstruct_backward(grad_out, ids, out, groups, True, members))
     t_linear_bwd, reps_grad = timed(lambda: hidden_grad @ weight)
-    t_mean_bwd, dx = timed(lambda: rt.cluster_mean_backward(reps_grad, ids, counts))
+    t_mean_bwd, dx = timed(lambda: rt.cluster_mean_backward(reps_grad, ids, counts, members))
     gb = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
     C = groups
     ops = {

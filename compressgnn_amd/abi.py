@@ -207,21 +207,23 @@ def cluster_mean(x, members, counts):
     return reps
 
 
-def cluster_mean_backward(grad, ids, counts):
+def cluster_mean_backward(grad, ids, counts, members=None):
     N = ids.numel()
     F = grad.shape[1]
     dx = torch.empty((N, F), dtype=grad.dtype, device=grad.device)
+    perm = None if members is None else members[1]
     check(lib().cgnn_cluster_mean_backward(i64(N), i64(F), i64(counts.numel()), dtype_code(grad.dtype),
-                                           ptr(grad), ptr(ids), ptr(counts), ptr(dx), stream_of(grad)))
+                                           ptr(grad), ptr(ids), ptr(counts), ptr(perm), ptr(dx), stream_of(grad)))
     return dx
 
 
-def reconstruct(reps, ids, bias=None, relu=False):
+def reconstruct(reps, ids, bias=None, relu=False, members=None):
     N = ids.numel()
     F = reps.shape[1]
     out = torch.empty((N, F), dtype=reps.dtype, device=reps.device)
+    perm = None if members is None else members[1]
     check(lib().cgnn_reconstruct(i64(N), i64(F), i64(reps.shape[0]), dtype_code(reps.dtype), ptr(reps),
-                                 ptr(ids), ptr(bias), ctypes.c_int(1 if relu else 0), ptr(out),
+                                 ptr(ids), ptr(perm), ptr(bias), ctypes.c_int(1 if relu else 0), ptr(out),
                                  stream_of(reps)))
     return out
 

@@ -25,7 +25,12 @@ namespace {
 // real column and are ignored when the code is formed.
 
 constexpr int kLshRows = 64;
-constexpr int kLshMaxSlab = 128;  // columns staged per pass (floats)
+constexpr int kLshMaxSlab = 32;  // columns staged per pass (floats): 9 KB of LDS per wave
+
+// One correctly rounded fused multiply-add in the operand type (the float overload must
+// not go through double: rounding twice is not the same operation).
+__device__ __forceinline__ float fused_mul_add(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fused_mul_add(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
 template <typename T>
 struct LshArgs {
@@ -76,16 +81,19 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_kernel(LshArgs<T> a) {
             const LPack<T, VEC> *mine = tile + lane * a.stride_v;
             for (int c = 0; c < ks_v; ++c) {
                 LPack<T, VEC> x = mine[c];
+                // all plane values of these VEC columns first (wave-uniform addresses:
+                // scalar loads issued back to back), then the multiply-add chains
+                T w[VEC][HB];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    const int k = k0 + c * VEC + i;
-                    const T *wrow = a.W + (int64_t)k * (EXACT ? HB : H);
+                    const T *wrow = a.W + (int64_t)(k0 + c * VEC + i) * (EXACT ? HB : H);
 #pragma unroll
-                    for (int j = 0; j < HB; ++j) {
-                        T w = EXACT ? wrow[j] : wrow[min(j, H - 1)];
-                        acc[j] = __builtin_fma(x.v[i], w, acc[j]);
-                    }
+                    for (int j = 0; j < HB; ++j) w[i][j] = EXACT ? wrow[j] : wrow[min(j, H - 1)];
                 }
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                    for (int j = 0; j < HB; ++j) acc[j] = fused_mul_add(x.v[i], w[i][j], acc[j]);
             }
         }
     }
@@ -271,11 +279,26 @@ struct GatherArgs {
     const T *__restrict__ src;       // [groups x F]
     const int64_t *__restrict__ ids; // [N]
     const int32_t *__restrict__ counts;
+    const int32_t *__restrict__ perm; // [N] or NULL: order in which the rows are produced
     const T *__restrict__ bias;
     T *__restrict__ out;             // [N x F]
     int64_t N, F, groups;
     int32_t relu;
 };
+
+// Output rows are written once and not read again here: streaming stores.
+template <typename T, int VEC>
+__device__ __forceinline__ void store_stream(T *p, const LPack<T, VEC> &x) {
+    if constexpr (VEC == 1) {
+        __builtin_nontemporal_store(x.v[0], p);
+    } else {
+        typedef T vec_t __attribute__((ext_vector_type(VEC)));
+        vec_t v;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = x.v[i];
+        __builtin_nontemporal_store(v, reinterpret_cast<vec_t *>(p));
+    }
+}
 
 template <typename T, int VEC, int LPR, int OP>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
@@ -283,11 +306,15 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
     const int lane = threadIdx.x % LPR;
     int64_t first = ((int64_t)blockIdx.x * GPB + threadIdx.x / LPR) * kGatherRows;
     if (first >= a.N) return;
-    int64_t g[kGatherRows];
+    // With `perm` (rows grouped by cluster) consecutive lane groups read the same row of
+    // src, which then comes from cache instead of memory; the result does not depend on
+    // the order.
+    int64_t g[kGatherRows], row[kGatherRows];
 #pragma unroll
     for (int r = 0; r < kGatherRows; ++r) {
-        int64_t i = first + r < a.N ? first + r : a.N - 1;
-        g[r] = a.ids[i];
+        const int64_t p = first + r < a.N ? first + r : a.N - 1;
+        row[r] = a.perm ? (int64_t)a.perm[p] : p;
+        g[r] = a.ids[row[r]];
     }
     T denom[kGatherRows];
     if constexpr (OP == GATHER_MEAN_GRAD) {
@@ -317,7 +344,7 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
                 }
                 x[r].v[i] = v;
             }
-            *reinterpret_cast<LPack<T, VEC> *>(a.out + (first + r) * a.F + f) = x[r];
+            store_stream<T, VEC>(a.out + row[r] * a.F + f, x[r]);
         }
     }
 }
@@ -385,7 +412,7 @@ cgnn_csr members_csr(int64_t N, int64_t groups, const int32_t *offsets, const in
     A.rowidx = sorted_id;
     A.val = nullptr;
     A.max_row_nnz = 0;
-    A.seg_nnz = 0;
+    A.seg_nnz = 256;  // clusters are often large: longer runs mean fewer carry rows to add up
     return A;
 }
 
@@ -491,12 +518,13 @@ extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype
 
 template <typename T, int OP>
 static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, const int64_t *ids,
-                        const int32_t *counts, const void *bias, int relu, void *out,
+                        const int32_t *counts, const int32_t *perm, const void *bias, int relu, void *out,
                         hipStream_t stream) {
     GatherArgs<T> a{};
     a.src = static_cast<const T *>(src);
     a.ids = ids;
     a.counts = counts;
+    a.perm = perm;
     a.bias = static_cast<const T *>(bias);
     a.out = static_cast<T *>(out);
     a.N = N;
@@ -508,27 +536,28 @@ static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, c
 
 extern "C" int cgnn_cluster_mean_backward(int64_t N, int64_t F, int64_t groups, int dtype,
                                           const void *grad, const int64_t *ids,
-                                          const int32_t *counts, void *dx, cgnn_stream_t stream) {
+                                          const int32_t *counts, const int32_t *perm, void *dx,
+                                          cgnn_stream_t stream) {
     CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 1, "cgnn_cluster_mean_backward: bad size");
     if (N == 0 || F == 0) return CGNN_OK;
     CGNN_REQUIRE(grad && ids && counts && dx, "cgnn_cluster_mean_backward: null array");
     if (dtype == CGNN_F32)
-        return gather_typed<float, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, nullptr, 0, dx, stream);
+        return gather_typed<float, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, perm, nullptr, 0, dx, stream);
     if (dtype == CGNN_F64)
-        return gather_typed<double, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, nullptr, 0, dx, stream);
+        return gather_typed<double, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, perm, nullptr, 0, dx, stream);
     return fail(CGNN_EUNSUPPORTED, "cgnn_cluster_mean_backward: dtype must be f32 or f64");
 }
 
 extern "C" int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
-                                const int64_t *ids, const void *bias, int relu, void *out,
-                                cgnn_stream_t stream) {
+                                const int64_t *ids, const int32_t *perm, const void *bias, int relu,
+                                void *out, cgnn_stream_t stream) {
     CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 0, "cgnn_reconstruct: bad size");
     if (N == 0 || F == 0) return CGNN_OK;
     CGNN_REQUIRE(reps && ids && out, "cgnn_reconstruct: null array");
     if (dtype == CGNN_F32)
-        return gather_typed<float, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, bias, relu, out, stream);
+        return gather_typed<float, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, relu, out, stream);
     if (dtype == CGNN_F64)
-        return gather_typed<double, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, bias, relu, out, stream);
+        return gather_typed<double, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, relu, out, stream);
     return fail(CGNN_EUNSUPPORTED, "cgnn_reconstruct: dtype must be f32 or f64");
 }
 

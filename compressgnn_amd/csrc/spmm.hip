@@ -311,44 +311,70 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
 }
 
 // Adds the carries of every row that straddles runs, in ascending run order, and
-// (when not accumulating) clears the rows that have no entries.  Work item i < nseg
-// handles run i if it is the first carry of its row; work item i < rows handles row i
-// if it is empty.  The two sets of rows are disjoint.
-template <typename T, int VEC, int LPR, int TILES>
+// (when not accumulating) clears the rows that have no entries.  One thread looks at
+// one work item: item i < nseg is run i, which matters if it holds the first carry of
+// its row; item i < rows is row i, which matters if it is empty (the two sets of rows
+// are disjoint).  The items that matter are then handled one after the other by the
+// whole wave, lanes across the features, with kFixBatch carry rows in flight.
+constexpr int kFixBatch = 8;
+
+template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
-    constexpr int GPB = kBlock / LPR;
-    const int lane = threadIdx.x % LPR;
-    int item = blockIdx.x * GPB + threadIdx.x / LPR;
-    if constexpr (LPR == kWave) item = __builtin_amdgcn_readfirstlane(item);
-    int64_t foff[TILES];
-    feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
-    Acc<T, VEC, TILES, MODE_UNIT> acc;
+    const int lane = threadIdx.x % kWave;
+    const int item = blockIdx.x * kBlock + threadIdx.x;
+    const int wave_item0 = item - lane;
+    int r = -1;
+    bool head = false;
     if (item < a.nseg) {
-        const int r = a.carry_row[item];
-        if (r >= 0 && (item == 0 || a.carry_row[item - 1] != r)) {
-            acc.clear();
-            int s = item;
-            do {
-                const T *crow = a.carry + (int64_t)s * a.F;
-                Pack<T, VEC> cval[TILES];
+        r = a.carry_row[item];
+        head = r >= 0 && (item == 0 || a.carry_row[item - 1] != r);
+    }
+    const bool empty = !a.accumulate && item < a.rows && a.rowptr[item] == a.rowptr[item + 1];
+    unsigned long long heads = __ballot(head);
+    while (heads) {
+        const int src = __ffsll(heads) - 1;
+        heads &= heads - 1;
+        const int row = __shfl(r, src, kWave);
+        const int s0 = wave_item0 + src;
+        for (int64_t f = (int64_t)lane * VEC; f < a.F; f += (int64_t)kWave * VEC) {
+            Pack<T, VEC> acc;
 #pragma unroll
-                for (int t = 0; t < TILES; ++t) {
-                    if (foff[t] >= 0) cval[t] = load_pack<T, VEC>(crow + foff[t]);
-                    else
+            for (int i = 0; i < VEC; ++i) acc.v[i] = T(0);
+            bool more = true;
+            for (int s = s0; more; s += kFixBatch) {
+                int rr[kFixBatch];
+                Pack<T, VEC> c[kFixBatch];
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) cval[t].v[i] = T(0);
+                for (int u = 0; u < kFixBatch; ++u) {
+                    const int idx = min(s + u, a.nseg - 1);
+                    rr[u] = a.carry_row[idx];
+                    c[u] = load_pack<T, VEC>(a.carry + (int64_t)idx * a.F + f);
                 }
-                acc.add(cval, T(1), 0);
-                ++s;
-            } while (s < a.nseg && a.carry_row[s] == r);
-            write_row<T, VEC, TILES, MODE_UNIT>(a.Y, a.F, r, foff, acc, 1);
+#pragma unroll
+                for (int u = 0; u < kFixBatch; ++u) {
+                    more = more && (s + u < a.nseg) && (rr[u] == row);
+                    if (more)
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
+                }
+            }
+            T *y = a.Y + (int64_t)row * a.F + f;
+            Pack<T, VEC> o = load_pack<T, VEC>(y);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) o.v[i] = o.v[i] + acc.v[i];
+            store_pack<T, VEC>(y, o);
         }
     }
-    if (!a.accumulate && item < a.rows) {
-        if (a.rowptr[item] == a.rowptr[item + 1]) {
-            acc.clear();
-            write_row<T, VEC, TILES, MODE_UNIT>(a.Y, a.F, item, foff, acc, 0);
-        }
+    unsigned long long empties = __ballot(empty);
+    while (empties) {
+        const int src = __ffsll(empties) - 1;
+        empties &= empties - 1;
+        const int row = wave_item0 + src;
+        Pack<T, VEC> zero;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) zero.v[i] = T(0);
+        for (int64_t f = (int64_t)lane * VEC; f < a.F; f += (int64_t)kWave * VEC)
+            store_pack_stream<T, VEC>(a.Y + (int64_t)row * a.F + f, zero);
     }
 }
 
@@ -421,7 +447,7 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_RELU_MASK>), grid, block, 0, stream, a);
             break;
         case KIND_FIXUP:
-            hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR, TILES>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC>), dim3((unsigned)ceil_div(items, kBlock)), block, 0, stream, a);
             break;
     }
     return check_launch("spmm launch");

@@ -455,7 +455,7 @@ Tensor cluster_mean(Tensor input, Tensor index, Tensor count, c10::optional<std:
 }
 
 // cluster_mean_backward_cuda (cluster_kernel.cu:171-181).
-Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count) {
+Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count, c10::optional<std::vector<Tensor>> members) {
     check_float(grad);
     check_index(index, grad.device());
     check_count(count, grad.device());
@@ -463,15 +463,23 @@ Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count) {
     c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
     Tensor out = torch::empty({index.numel(), grad.size(1)}, grad.options());
     if (out.numel() == 0) return out;
+    const int32_t *perm = nullptr;
+    if (members.has_value() && !members->empty()) {
+        TORCH_CHECK(members->size() == 3 && (*members)[1].numel() == index.numel() &&
+                        (*members)[1].scalar_type() == torch::kInt32 && (*members)[1].device() == index.device(),
+                    "member lists do not match index");
+        perm = (*members)[1].data_ptr<int32_t>();
+    }
     ok(cgnn_cluster_mean_backward(index.numel(), grad.size(1), count.numel(), dtype_code(grad), grad.data_ptr(),
-                                  index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), out.data_ptr(),
+                                  index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), perm, out.data_ptr(),
                                   current_stream(grad)),
        "cluster_mean_backward");
     return out;
 }
 
 // cluster_reconstruct_cuda (cluster_kernel.cu:182-195).
-Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias, bool relu) {
+Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias, bool relu,
+                           c10::optional<std::vector<Tensor>> members) {
     check_float(reps);
     check_index(index, reps.device());
     if (bias.has_value())
@@ -481,8 +489,15 @@ Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias
     c10::hip::HIPGuardMasqueradingAsCUDA guard(reps.device());
     Tensor out = torch::empty({index.numel(), reps.size(1)}, reps.options());
     if (out.numel() == 0) return out;
+    const int32_t *perm = nullptr;
+    if (members.has_value() && !members->empty()) {
+        TORCH_CHECK(members->size() == 3 && (*members)[1].numel() == index.numel() &&
+                        (*members)[1].scalar_type() == torch::kInt32 && (*members)[1].device() == index.device(),
+                    "member lists do not match index");
+        perm = (*members)[1].data_ptr<int32_t>();
+    }
     ok(cgnn_reconstruct(index.numel(), reps.size(1), reps.size(0), dtype_code(reps), reps.data_ptr(),
-                        index.data_ptr<int64_t>(), bias.has_value() ? bias->data_ptr() : nullptr, relu ? 1 : 0,
+                        index.data_ptr<int64_t>(), perm, bias.has_value() ? bias->data_ptr() : nullptr, relu ? 1 : 0,
                         out.data_ptr(), current_stream(reps)),
        "cluster_reconstruct");
     return out;
@@ -524,8 +539,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("cluster_assign", &cluster_assign);
     m.def("cluster_mean", &cluster_mean, py::arg("input"), py::arg("index"), py::arg("count"),
           py::arg("members") = py::none());
-    m.def("cluster_mean_backward", &cluster_mean_backward);
-    m.def("cluster_reconstruct", &cluster_reconstruct);
+    m.def("cluster_mean_backward", &cluster_mean_backward, py::arg("grad"), py::arg("index"), py::arg("count"),
+          py::arg("members") = py::none());
+    m.def("cluster_reconstruct", &cluster_reconstruct, py::arg("reps"), py::arg("index"), py::arg("bias"),
+          py::arg("relu"), py::arg("members") = py::none());
     m.def("cluster_reconstruct_backward", &cluster_reconstruct_backward, py::arg("grad"), py::arg("index"),
           py::arg("output"), py::arg("groups"), py::arg("relu"), py::arg("members") = py::none());
     // additions of this build

@@ -66,7 +66,7 @@ def _mean_forward(x, index, counts):
 
 def _mean_backward(grad, index, counts):
     """reference layer/CompressgnnCluster.py:22-25"""
-    return _native.cluster_mean_backward(grad.contiguous(), index, counts)
+    return _native.cluster_mean_backward(grad.contiguous(), index, counts, members_of(index, counts.numel()))
 
 
 class _Mean(torch.autograd.Function):

@@ -15,10 +15,11 @@ class _Reconstruct(torch.autograd.Function):
     @staticmethod
     def forward(ctx, src, index, bias, relu):
         index = index.contiguous()
-        output = _native.cluster_reconstruct(src.contiguous(), index, None if bias is None else bias.contiguous(), relu)
+        ctx.members = members_of(index, src.size(0))
+        output = _native.cluster_reconstruct(src.contiguous(), index, None if bias is None else bias.contiguous(),
+                                             relu, ctx.members)
         ctx.save_for_backward(index, output)
         ctx.groups, ctx.relu, ctx.has_bias = src.size(0), relu, bias is not None
-        ctx.members = members_of(index, src.size(0))
         return output
 
     @staticmethod

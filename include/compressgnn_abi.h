@@ -149,17 +149,20 @@ int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype, const voi
                       const int32_t *counts, void *reps, void *workspace,
                       size_t workspace_bytes, cgnn_stream_t stream);
 
-/* dx[i,:] = grad[ids[i],:] / max(counts[ids[i]],1).
+/* dx[i,:] = grad[ids[i],:] / max(counts[ids[i]],1).  perm (the member list of
+ * cgnn_cluster_members for these ids, or NULL) only sets the order in which rows are
+ * produced: grouped by cluster, every row of grad is fetched from memory once.
  * Replaces cluster_mean_backward_cuda (cluster_kernel.cu:171-181). */
 int cgnn_cluster_mean_backward(int64_t N, int64_t F, int64_t groups, int dtype, const void *grad,
-                               const int64_t *ids, const int32_t *counts, void *dx,
-                               cgnn_stream_t stream);
+                               const int64_t *ids, const int32_t *counts, const int32_t *perm,
+                               void *dx, cgnn_stream_t stream);
 
 /* out[i,:] = act(reps[ids[i],:] + bias), act(v) = (relu && v < 0) ? 0 : v; bias may be
- * NULL.  Replaces cluster_reconstruct_cuda (cluster_kernel.cu:182-195). */
+ * NULL; perm as above (NULL = rows in natural order).
+ * Replaces cluster_reconstruct_cuda (cluster_kernel.cu:182-195). */
 int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
-                     const int64_t *ids, const void *bias, int relu, void *out,
-                     cgnn_stream_t stream);
+                     const int64_t *ids, const int32_t *perm, const void *bias, int relu,
+                     void *out, cgnn_stream_t stream);
 
 /* reps_grad[g,:] = sum over members i of g (ascending) of
  * ((relu && output[i,:] <= 0) ? 0 : grad[i,:]).

@@ -47,7 +47,7 @@ class OracleNative:
         return torch.from_numpy(oracle.cluster_mean(x.detach().numpy(), index.numpy(), counts.numpy()))
 
     @staticmethod
-    def cluster_mean_backward(grad, index, counts):
+    def cluster_mean_backward(grad, index, counts, members=None):
         return torch.from_numpy(oracle.cluster_mean_backward(grad.numpy(), index.numpy(), counts.numpy()))
 
 

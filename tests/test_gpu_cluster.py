@@ -52,14 +52,17 @@ def test_assign_mean_reconstruct(dtype, width, n, bits):
     assert_within(reps, want_reps, **tol)
     assert np.array_equal(reps[small], want_reps[small])
     grad = rng.standard_normal((groups, width)).astype(dtype)
-    dx = abi.cluster_mean_backward(_t(grad), ids, counts)
-    assert np.array_equal(dx.cpu().numpy(), oracle.cluster_mean_backward(grad, want_ids, want_counts))
+    want_dx = oracle.cluster_mean_backward(grad, want_ids, want_counts)
+    assert np.array_equal(abi.cluster_mean_backward(_t(grad), ids, counts).cpu().numpy(), want_dx)
+    assert np.array_equal(abi.cluster_mean_backward(_t(grad), ids, counts, members).cpu().numpy(), want_dx)
     bias = rng.standard_normal(width).astype(dtype)
     for relu in (False, True):
         for b in (None, bias):
             out = abi.reconstruct(_t(grad), ids, None if b is None else _t(b), relu)
             want = oracle.reconstruct(grad, want_ids, b, relu)
             assert np.array_equal(out.cpu().numpy(), want)
+            grouped = abi.reconstruct(_t(grad), ids, None if b is None else _t(b), relu, members)
+            assert np.array_equal(grouped.cpu().numpy(), want)  # row order does not change the result
             go = rng.standard_normal((n, width)).astype(dtype)
             rg = abi.reconstruct_backward(_t(go), out, members, groups, relu).cpu().numpy()
             want_rg = oracle.reconstruct_backward(go, want_ids, want, groups, relu)
