@@ -412,7 +412,7 @@ cgnn_csr members_csr(int64_t N, int64_t groups, const int32_t *offsets, const in
     A.rowidx = sorted_id;
     A.val = nullptr;
     A.max_row_nnz = 0;
-    A.seg_nnz = 256;  // clusters are often large: longer runs mean fewer carry rows to add up
+    A.seg_nnz = 0;  // default run length: measured best for both cluster sums
     return A;
 }
 
@@ -524,7 +524,8 @@ static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, c
     a.src = static_cast<const T *>(src);
     a.ids = ids;
     a.counts = counts;
-    a.perm = perm;
+    // scattered row writes pay off only when a row is a whole number of 128-byte lines
+    a.perm = (F * (int64_t)sizeof(T)) % 128 == 0 ? perm : nullptr;
     a.bias = static_cast<const T *>(bias);
     a.out = static_cast<T *>(out);
     a.N = N;

@@ -314,13 +314,29 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
 // (when not accumulating) clears the rows that have no entries.  One thread looks at
 // one work item: item i < nseg is run i, which matters if it holds the first carry of
 // its row; item i < rows is row i, which matters if it is empty (the two sets of rows
-// are disjoint).  The items that matter are then handled one after the other by the
-// whole wave, lanes across the features, with kFixBatch carry rows in flight.
+// are disjoint).  The items of a wave that matter are then dealt out to its lane groups
+// (LPR lanes across the features), kFixBatch carry rows in flight per group.
 constexpr int kFixBatch = 8;
 
-template <typename T, int VEC>
+// Lane (within the wave) of the flagged item this lane's group should handle in the
+// round that starts at rank `base`, or -1.  Uniform control flow: every lane calls it.
+template <int LPR>
+__device__ __forceinline__ int deal_item(bool flag, int my_rank, int base, int grp) {
+    constexpr int G = kWave / LPR;
+    int src = -1;
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+        const unsigned long long m = __ballot(flag && my_rank == base + gi);
+        if (gi == grp && m) src = __ffsll(m) - 1;
+    }
+    return src;
+}
+
+template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
+    constexpr int G = kWave / LPR;
     const int lane = threadIdx.x % kWave;
+    const int sub = lane % LPR, grp = lane / LPR;
     const int item = blockIdx.x * kBlock + threadIdx.x;
     const int wave_item0 = item - lane;
     int r = -1;
@@ -330,13 +346,16 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
         head = r >= 0 && (item == 0 || a.carry_row[item - 1] != r);
     }
     const bool empty = !a.accumulate && item < a.rows && a.rowptr[item] == a.rowptr[item + 1];
-    unsigned long long heads = __ballot(head);
-    while (heads) {
-        const int src = __ffsll(heads) - 1;
-        heads &= heads - 1;
-        const int row = __shfl(r, src, kWave);
+    const unsigned long long below = (1ull << lane) - 1ull;
+
+    const unsigned long long heads = __ballot(head);
+    const int n_heads = __popcll(heads), head_rank = __popcll(heads & below);
+    for (int base = 0; base < n_heads; base += G) {
+        const int src = deal_item<LPR>(head, head_rank, base, grp);
+        const int row = __shfl(r, src < 0 ? 0 : src, kWave);
+        if (src < 0) continue;
         const int s0 = wave_item0 + src;
-        for (int64_t f = (int64_t)lane * VEC; f < a.F; f += (int64_t)kWave * VEC) {
+        for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC) {
             Pack<T, VEC> acc;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc.v[i] = T(0);
@@ -365,15 +384,17 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
             store_pack<T, VEC>(y, o);
         }
     }
-    unsigned long long empties = __ballot(empty);
-    while (empties) {
-        const int src = __ffsll(empties) - 1;
-        empties &= empties - 1;
+
+    const unsigned long long empties = __ballot(empty);
+    const int n_empty = __popcll(empties), empty_rank = __popcll(empties & below);
+    for (int base = 0; base < n_empty; base += G) {
+        const int src = deal_item<LPR>(empty, empty_rank, base, grp);
+        if (src < 0) continue;
         const int row = wave_item0 + src;
         Pack<T, VEC> zero;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) zero.v[i] = T(0);
-        for (int64_t f = (int64_t)lane * VEC; f < a.F; f += (int64_t)kWave * VEC)
+        for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC)
             store_pack_stream<T, VEC>(a.Y + (int64_t)row * a.F + f, zero);
     }
 }
@@ -447,7 +468,7 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_RELU_MASK>), grid, block, 0, stream, a);
             break;
         case KIND_FIXUP:
-            hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC>), dim3((unsigned)ceil_div(items, kBlock)), block, 0, stream, a);
+            hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, kBlock)), block, 0, stream, a);
             break;
     }
     return check_launch("spmm launch");
