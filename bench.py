@@ -40,6 +40,19 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def recorded_traffic():
+    """HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc runs
+    summarised in profiles/ (FETCH_SIZE and WRITE_SIZE scaled by the copy-kernel probe)."""
+    path = os.path.join(ROOT, "profiles", "spmm_nnz_dual_C1_F128_pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch"):
+                return int(float(line.split("=")[1]))
+    except OSError:
+        pass
+    return None
+
+
 def block_bytes(rowptr, col, ncols, F, acc, elt=4):
     """Algorithmic bytes of one CSR product: indices + values (8 B per non-zero), row
     pointers, every gathered input row once, every non-empty output row once (twice when
@@ -406,9 +419,9 @@ def main():
                                "sym-norm), compressed propagation forward + backward, F=%d fp32" % (len(e_raw), F),
                    "rules": int(data.rule_cnt), "levels": int(graph.step)},
         "frac_of_hbm_peak": value / HBM_PEAK_GBPS,
-        "roofline": {"bound": "hbm", "kernel": "spmm_pair_kernel (forward vertex stage: v2r + v2v fused)",
+        "roofline": {"bound": "hbm", "kernel": "cgnn_spmm_dual, forward vertex stage [v2v | v2r]: spmm_nnz_kernel<float,4,32,1,dual> + its fix-up pass",
                      "achieved": dom_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom_gbps / HBM_PEAK_GBPS,
-                     "traffic": None, "ms": dom, "bytes": dom_bytes},
+                     "traffic": recorded_traffic(), "ms": dom, "bytes": dom_bytes},
         "cpu_baseline": cpu,
         "detail": detail,
     }
