@@ -2,6 +2,8 @@
 // histogram, occupancy scan, id remap, row gathers (mean backward, reconstruct with
 // fused bias + ReLU).  The per-cluster sums (mean forward, reconstruct backward) run
 // on the member lists through the nnz-schedule SpMM in spmm.hip.
+#include <type_traits>
+
 #include "common.h"
 
 namespace cgnn {
@@ -13,16 +15,16 @@ namespace {
 
 // ------------------------------------------------------------------ LSH hash ---
 //
-// One lane per row, one wave (64 rows) per workgroup.  The wave stages its 64 rows
-// of X, KS columns at a time, in LDS with fully coalesced 16-byte loads, then every
-// lane walks its own row: h_j = fma(x_k, W[k,j], h_j) for k ascending, which fixes
-// the rounding of every projection (the CPU oracle uses the same chain).  W is read
-// with wave-uniform addresses, i.e. through the scalar unit, so the inner loop is one
-// LDS read per 4 k and HB vector FMAs per k.  The LDS row stride is odd in units of
-// the access width, which keeps the 64 strided row reads free of bank conflicts.
+// Every projection is the chain h_j = fma(x_k, W[k,j], h_j) for k ascending from 0, which
+// fixes its rounding (the CPU oracle uses the same chain).  Tiles of 64 rows of X are
+// staged in LDS with coalesced 16-byte loads; the LDS row stride is odd in units of the
+// access width, which keeps the 64 strided row reads free of bank conflicts.
 //
-// HB = number of accumulators (bits rounded up); columns >= bits repeat the last
-// real column and are ignored when the code is formed.
+// Vector-unit kernel (used for double precision): one lane per row, one wave per
+// workgroup, KS columns per pass.  W is read with wave-uniform addresses, i.e. through the
+// scalar unit, so the inner loop is one LDS read per pack of k and HB vector FMAs per k.
+// HB = number of accumulators (bits rounded up); columns >= bits repeat the last real
+// column and are ignored when the code is formed.
 
 constexpr int kLshRows = 64;
 constexpr int kLshMaxSlab = 32;  // columns staged per pass (floats): 9 KB of LDS per wave
@@ -43,6 +45,7 @@ struct LshArgs {
     int32_t bits;
     int32_t slab;      // columns per pass, multiple of VEC
     int32_t stride_v;  // LDS row stride in units of VEC elements (odd)
+    int32_t wstride;   // matrix-unit kernel, 16-byte rows: LDS stride of a plane in floats
     uint32_t magic;    // floor(2^32 / slab_v) + 1: i / slab_v == mulhi(i, magic) for i < 2^16
 };
 
@@ -107,6 +110,307 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_kernel(LshArgs<T> a) {
     }
 }
 
+// Single precision runs the same chains on the matrix unit.  v_mfma_f32_16x16x1_4b_f32
+// computes, for four independent 16x16 blocks, D[i][j] = fma(A[i], B[j], C[i][j]) with
+// one rounding (K = 1, so no sum is formed inside the instruction; results agree bit
+// for bit with fmaf, denormals included).  Lane L supplies A = x[row L][k] (block L/16,
+// i = L%16) and B = W[k][L%16]; one instruction advances all 64 rows x 16 planes by
+// one k at twice the rate of 16 vector FMAs and without touching the scalar unit.
+// Accumulator register v of lane L holds plane L%16 of row 16*(v/4) + 4*(L/16) + v%4,
+// so ballot(acc[v] > 0) carries four complete 16-bit sign masks, one per 16-lane field.
+//
+// A pass stages up to 128 columns of the 64 rows, so rows of up to 512 bytes are read
+// whole and every cache line of X is fetched once.  That much LDS per wave leaves room for
+// only a few waves per compute unit, so the waves are persistent (each walks tiles
+// t, t + stride, ...) and keep the next pass in registers, in flight, while they multiply
+// the current one out of LDS.  W is staged with zero columns beyond `bits`; NG = 2 covers
+// 17..30 planes with two instructions per k.  lsh_hash_mfma_kernel is the general form
+// (any F, several passes per tile); lsh_hash_mfma_flat_kernel below is the form for
+// 16-byte-aligned rows of at most 128 columns.
+
+typedef float lsh_acc_t __attribute__((ext_vector_type(16)));
+typedef float lsh_f4_t __attribute__((ext_vector_type(4)));
+
+// Register / LDS element of the staged X tile: a native vector, so that the prefetch
+// array stays in registers.
+template <int VEC> struct LshPack;
+template <> struct LshPack<4> {
+    using type = lsh_f4_t;
+    static __device__ __forceinline__ float at(const type &p, int i) { return p[i]; }
+};
+template <> struct LshPack<1> {
+    using type = float;
+    static __device__ __forceinline__ float at(const type &p, int) { return p; }
+};
+
+constexpr int kLshMfmaSlab = 128;  // columns per pass: rows of up to 512 bytes are staged whole
+
+// Orders a wave's LDS writes before its own later reads of a region no other wave
+// touches.  The LDS unit executes the instructions of one wave in order, so only the
+// compiler has to be held; unlike a workgroup barrier this does not wait for global loads
+// and atomics in flight.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int VEC, int NG>
+__global__ __launch_bounds__(kLshRows) void lsh_hash_mfma_kernel(LshArgs<float> a, int64_t tiles) {
+    using Pack = typename LshPack<VEC>::type;
+    constexpr int HBP = 16 * NG;
+    constexpr int XPER = (VEC == 4 ? kLshMfmaSlab : kLshMaxSlab) / VEC;  // X packs per lane and pass
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    Pack *tile = reinterpret_cast<Pack *>(lds_raw);
+    float *wtile = reinterpret_cast<float *>(lds_raw + (size_t)kLshRows * a.stride_v * sizeof(Pack));
+    const int lane = threadIdx.x;
+    const int H = a.bits;
+    const int slabs = (a.F + a.slab - 1) / a.slab;
+
+    lsh_acc_t acc[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[g][v] = 0.f;
+
+    // columns [k0, k0 + slab) of the 64 rows of tile t: global -> registers, registers -> LDS
+    Pack xr[XPER];
+    auto fetch = [&](int64_t t, int k0) {
+        const int64_t row0 = t * kLshRows;
+        const int rows_here = (int)min((int64_t)kLshRows, a.N - row0);
+        const float *xbase = a.X + row0 * (int64_t)a.F + k0;
+        const int ks_v = min(a.slab, a.F - k0) / VEC;
+        const bool full = ks_v * VEC == a.slab && a.magic != 0;
+        const int total = rows_here * ks_v;
+#pragma unroll
+        for (int u = 0; u < XPER; ++u) {
+            const int i = lane + u * kLshRows;
+            if (i < total) {
+                const int r = full ? (int)__umulhi((uint32_t)i, a.magic) : i / ks_v;
+                const int c = i - r * ks_v;
+                xr[u] = *reinterpret_cast<const Pack *>(xbase + (int64_t)r * a.F + c * VEC);
+            }
+        }
+    };
+    auto commit = [&](int64_t t, int k0) {
+        const int rows_here = (int)min((int64_t)kLshRows, a.N - t * kLshRows);
+        const int ks_v = min(a.slab, a.F - k0) / VEC;
+        const bool full = ks_v * VEC == a.slab && a.magic != 0;
+        const int total = rows_here * ks_v;
+#pragma unroll
+        for (int u = 0; u < XPER; ++u) {
+            const int i = lane + u * kLshRows;
+            if (i < total) {
+                const int r = full ? (int)__umulhi((uint32_t)i, a.magic) : i / ks_v;
+                const int c = i - r * ks_v;
+                tile[r * a.stride_v + c] = xr[u];
+            }
+        }
+    };
+    // planes k0 .. k0+slab, zero beyond `bits`: [plane][k] with row stride wstride for
+    // 16-byte reads of four consecutive k (VEC == 4), else [k][16*NG]
+    auto stage_planes = [&](int k0) {
+        const int n = min(a.slab, a.F - k0) * HBP;
+        for (int e = lane; e < n; e += kLshRows) {
+            const int kk = e / HBP, j = e % HBP;
+            const float w = j < H ? a.W[(int64_t)(k0 + kk) * H + j] : 0.f;
+            wtile[VEC == 4 ? j * a.wstride + kk : e] = w;
+        }
+    };
+
+    // The wave walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...; while it multiplies
+    // one pass out of LDS, the next pass (of this tile or of the next one) is in flight.
+    const int myv = 4 * (lane >> 4) + (lane & 3);
+    if (slabs == 1) stage_planes(0);  // same planes for every tile; ordered before the first pass's reads
+    fetch(blockIdx.x, 0);
+    for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+        for (int s = 0; s < slabs; ++s) {
+            const int k0 = s * a.slab;
+            const int ks_v = min(a.slab, a.F - k0) / VEC;
+            wave_lds_sync();  // the previous pass has been consumed
+            commit(t, k0);
+            if (slabs > 1) stage_planes(k0);
+            wave_lds_sync();
+            if (s + 1 < slabs)
+                fetch(t, k0 + a.slab);
+            else if (t + gridDim.x < tiles)
+                fetch(t + gridDim.x, 0);
+            // rows beyond the end of X multiply stale LDS contents; a row of D depends on
+            // its own A element only, and those rows are never written out
+            const Pack *mine = tile + lane * a.stride_v;
+            if constexpr (VEC == 4) {
+                const lsh_f4_t *wq = reinterpret_cast<const lsh_f4_t *>(wtile + (lane & 15) * a.wstride);
+                const int gstep = 4 * a.wstride;  // 16 planes further, in 16-byte units
+#pragma unroll 4
+                for (int c = 0; c < ks_v; ++c) {
+                    const lsh_f4_t x = mine[c];
+                    lsh_f4_t w[NG];
+#pragma unroll
+                    for (int g = 0; g < NG; ++g) w[g] = wq[g * gstep + c];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int g = 0; g < NG; ++g)
+                            acc[g] = __builtin_amdgcn_mfma_f32_16x16x1f32(x[i], w[g][i], acc[g], 0, 0, 0);
+                }
+            } else {
+                const float *wcol = wtile + (lane & 15);
+#pragma unroll 4
+                for (int c = 0; c < ks_v; ++c) {
+                    const float x = mine[c];
+#pragma unroll
+                    for (int g = 0; g < NG; ++g)
+                        acc[g] = __builtin_amdgcn_mfma_f32_16x16x1f32(x, wcol[c * HBP + g * 16], acc[g], 0, 0, 0);
+                }
+            }
+        }
+
+        unsigned long long sel[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            sel[g] = 0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const unsigned long long b = __ballot(acc[g][v] > 0.f);
+                sel[g] = myv == v ? b : sel[g];
+                acc[g][v] = 0.f;
+            }
+        }
+        const int64_t row = t * kLshRows + lane;
+        if (row < a.N) {
+            const int shift = 16 * ((lane & 15) >> 2);
+            uint32_t mask = (uint32_t)(sel[0] >> shift) & 0xffffu;  // bit j = (h_j > 0)
+            if (NG == 2) mask |= ((uint32_t)(sel[NG - 1] >> shift) & 0xffffu) << 16;
+            const int code = (int)(__brev(mask) >> (32 - H));  // plane 0 is the top bit
+            a.raw_code[row] = code;
+            atomicAdd(a.bucket_count + code, 1);
+        }
+    }
+}
+
+// Whole rows per pass (F <= 128, 16-byte packs): the 64 rows of a tile are one contiguous
+// range of X, so pack p = lane + 64*u of the tile needs no index arithmetic on the way in
+// and a lane moves exactly F/4 packs per tile.  XP >= F/4 packs are loaded without any
+// branch (offsets clamped to the last pack of the tile, which also covers the partial last
+// tile: the rows such loads fill are not written out); only the LDS writes are guarded, by
+// a wave-uniform condition.  The code of a tile is stored (and its bucket counted) only
+// after the next tile has been committed to LDS, so that no wait for the loads also waits
+// for that atomic.
+constexpr int kLshFlatMaxWaves = 8;
+
+template <int NG, int XP>
+__global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat_kernel(LshArgs<float> a,
+                                                                                       int64_t tiles) {
+    // LDS: the planes, shared by the waves of the workgroup, then one X tile per wave.
+    // The waves are independent after the planes have been staged.
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int lane = threadIdx.x & (kLshRows - 1);
+    const int wave = threadIdx.x / kLshRows;
+    const int waves = blockDim.x / kLshRows;
+    float *wtile = reinterpret_cast<float *>(lds_raw);
+    lsh_f4_t *tile = reinterpret_cast<lsh_f4_t *>(lds_raw + (size_t)a.wstride * 16 * NG * sizeof(float)) +
+                     (size_t)wave * kLshRows * a.stride_v;
+    const int H = a.bits;
+    const int ks_v = a.F / 4;  // packs per row = packs per lane and tile
+    const lsh_f4_t *X4 = reinterpret_cast<const lsh_f4_t *>(a.X);
+    const int64_t first = (int64_t)blockIdx.x * waves + wave;
+    const int64_t step = (int64_t)gridDim.x * waves;
+
+    for (int e = threadIdx.x; e < a.F * 16 * NG; e += blockDim.x) {  // planes as [plane][k]
+        const int kk = e / (16 * NG), j = e % (16 * NG);
+        wtile[j * a.wstride + kk] = j < H ? a.W[(int64_t)kk * H + j] : 0.f;
+    }
+    __syncthreads();
+
+    lsh_acc_t acc[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[g][v] = 0.f;
+
+    lsh_f4_t xr[XP];
+    auto fetch = [&](int64_t t) {
+        const int64_t row0 = t * kLshRows;
+        const lsh_f4_t *src = X4 + row0 * ks_v;
+        const int top = (int)min((int64_t)kLshRows, a.N - row0) * ks_v - 1;
+#pragma unroll
+        for (int u = 0; u < XP; ++u) xr[u] = __builtin_nontemporal_load(src + min(lane + u * kLshRows, top));
+    };
+    // slot of pack p: row * stride_v + column pack = p + row * (stride_v - ks_v)
+    const bool padded = a.stride_v != ks_v;
+    const int myv = 4 * (lane >> 4) + (lane & 3);
+    const int shift = 16 * ((lane & 15) >> 2);
+    const lsh_f4_t *mine = tile + lane * a.stride_v;
+    const lsh_f4_t *wq = reinterpret_cast<const lsh_f4_t *>(wtile + (lane & 15) * a.wstride);
+    const int gstep = 4 * a.wstride;  // 16 planes further, in 16-byte units
+
+    auto multiply = [&](int c, auto count) {
+        constexpr int n = decltype(count)::value;
+        lsh_f4_t x[n], w[NG][n];
+#pragma unroll
+        for (int i = 0; i < n; ++i) {
+            x[i] = mine[c + i];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) w[g][i] = wq[g * gstep + c + i];
+        }
+#pragma unroll
+        for (int i = 0; i < n; ++i)
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int g = 0; g < NG; ++g)
+                    acc[g] = __builtin_amdgcn_mfma_f32_16x16x1f32(x[i][k], w[g][i][k], acc[g], 0, 0, 0);
+    };
+
+    int pending_code = 0;
+    int64_t pending_row = -1;
+    if (first < tiles) fetch(first);
+    for (int64_t t = first; t < tiles; t += step) {
+        wave_lds_sync();  // the previous tile has been consumed
+#pragma unroll
+        for (int u = 0; u < XP; ++u) {
+            const int p = lane + u * kLshRows;
+            if (u < ks_v) tile[p + (padded ? (int)__umulhi((uint32_t)p, a.magic) : 0)] = xr[u];
+        }
+        wave_lds_sync();
+        if (pending_row >= 0 && pending_row < a.N) {
+            a.raw_code[pending_row] = pending_code;
+            atomicAdd(a.bucket_count + pending_code, 1);
+        }
+        if (t + step < tiles) fetch(t + step);
+
+        // eight column packs at a time: all sixteen LDS reads are issued before the first
+        // multiply, so their latency is paid once per 32 matrix instructions
+        int c = 0;
+        for (; c + 8 <= ks_v; c += 8) multiply(c, std::integral_constant<int, 8>{});
+        if (c + 4 <= ks_v) {
+            multiply(c, std::integral_constant<int, 4>{});
+            c += 4;
+        }
+        for (; c < ks_v; ++c) multiply(c, std::integral_constant<int, 1>{});
+
+        unsigned long long sel[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            sel[g] = 0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const unsigned long long b = __ballot(acc[g][v] > 0.f);
+                sel[g] = myv == v ? b : sel[g];
+                acc[g][v] = 0.f;
+            }
+        }
+        uint32_t mask = (uint32_t)(sel[0] >> shift) & 0xffffu;  // bit j = (h_j > 0)
+        if (NG == 2) mask |= ((uint32_t)(sel[NG - 1] >> shift) & 0xffffu) << 16;
+        pending_code = (int)(__brev(mask) >> (32 - H));  // plane 0 is the top bit
+        pending_row = t * kLshRows + lane;
+    }
+    if (pending_row >= 0 && pending_row < a.N) {
+        a.raw_code[pending_row] = pending_code;
+        atomicAdd(a.bucket_count + pending_code, 1);
+    }
+}
+
 // bits == 0 or F == 0: every projection is empty, code 0.
 __global__ void lsh_trivial_kernel(int32_t *raw_code, int32_t *bucket_count, int64_t N) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -137,14 +441,100 @@ int launch_lsh(const LshArgs<T> &a, hipStream_t stream) {
     return check_launch("lsh_hash");
 }
 
+// Compute units of the current device (looked up once per device).
+int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+template <typename Kernel>
+int launch_lsh_persistent(Kernel kernel, int waves, size_t lds, const LshArgs<float> &a, hipStream_t stream) {
+    const int64_t tiles = ceil_div(a.N, kLshRows);
+    // exactly as many workgroups as are resident at once, each wave walking its share of
+    // the tiles
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kLshRows * waves, lds) != hipSuccess ||
+        per_cu < 1)
+        per_cu = 1;
+    int64_t blocks = (int64_t)per_cu * compute_units();
+    if (blocks > ceil_div(tiles, waves)) blocks = ceil_div(tiles, waves);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kLshRows * waves), lds, stream, a, tiles);
+    return check_launch("lsh_hash");
+}
+
+constexpr size_t kLdsPerCu = 160 * 1024;
+constexpr size_t kLdsDefaultLimit = 64 * 1024;  // larger workgroups must be allowed per kernel
+
+template <int NG, int XP>
+int launch_lsh_flat(const LshArgs<float> &a, hipStream_t stream) {
+    const size_t tile_bytes = (size_t)kLshRows * a.stride_v * sizeof(lsh_f4_t);
+    const size_t plane_bytes = (size_t)a.wstride * 16 * NG * sizeof(float);
+    // as many waves as fit beside one copy of the planes; two per SIMD at most (registers)
+    int waves = (int)((kLdsPerCu - plane_bytes) / tile_bytes);
+    waves = waves < 1 ? 1 : (waves > kLshFlatMaxWaves ? kLshFlatMaxWaves : waves);
+    auto kernel = lsh_hash_mfma_flat_kernel<NG, XP>;
+    size_t lds = plane_bytes + waves * tile_bytes;
+    if (lds > kLdsDefaultLimit) {
+        static bool allowed = false, refused = false;  // per kernel instantiation
+        if (!allowed && !refused) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerCu) == hipSuccess)
+                allowed = true;
+            else {
+                refused = true;
+                (void)hipGetLastError();
+            }
+        }
+        if (!allowed) {
+            waves = (int)((kLdsDefaultLimit - plane_bytes) / tile_bytes);
+            waves = waves < 1 ? 1 : waves;
+            lds = plane_bytes + waves * tile_bytes;
+        }
+    }
+    return launch_lsh_persistent(kernel, waves, lds, a, stream);
+}
+
+template <int VEC, int NG>
+int launch_lsh_mfma(const LshArgs<float> &a, hipStream_t stream) {
+    if (VEC == 4 && a.slab == a.F) {  // whole rows per pass
+        const int packs = a.F / 4;
+        if (packs <= 4) return launch_lsh_flat<NG, 4>(a, stream);
+        if (packs <= 8) return launch_lsh_flat<NG, 8>(a, stream);
+        if (packs <= 12) return launch_lsh_flat<NG, 12>(a, stream);
+        if (packs <= 16) return launch_lsh_flat<NG, 16>(a, stream);
+        if (packs <= 20) return launch_lsh_flat<NG, 20>(a, stream);
+        if (packs <= 24) return launch_lsh_flat<NG, 24>(a, stream);
+        if (packs == 25) return launch_lsh_flat<NG, 25>(a, stream);
+        if (packs <= 28) return launch_lsh_flat<NG, 28>(a, stream);
+        return launch_lsh_flat<NG, 32>(a, stream);
+    }
+    const size_t x_bytes = (size_t)kLshRows * a.stride_v * VEC * sizeof(float);
+    return launch_lsh_persistent(lsh_hash_mfma_kernel<VEC, NG>, 1,
+                                 x_bytes + (size_t)(VEC == 4 ? a.wstride : a.slab) * 16 * NG * sizeof(float), a,
+                                 stream);
+}
+
 template <typename T, int VEC>
 int dispatch_lsh(const LshArgs<T> &a, hipStream_t stream) {
     const int H = a.bits;
-    if (H == 8) return launch_lsh<T, VEC, 8, true>(a, stream);
-    if (H == 16) return launch_lsh<T, VEC, 16, true>(a, stream);
-    if (H < 8) return launch_lsh<T, VEC, 8, false>(a, stream);
-    if (H < 16) return launch_lsh<T, VEC, 16, false>(a, stream);
-    return launch_lsh<T, VEC, 32, false>(a, stream);
+    if constexpr (sizeof(T) == sizeof(float)) {
+        if (H <= 16) return launch_lsh_mfma<VEC, 1>(a, stream);
+        return launch_lsh_mfma<VEC, 2>(a, stream);
+    } else {
+        if (H == 8) return launch_lsh<T, VEC, 8, true>(a, stream);
+        if (H == 16) return launch_lsh<T, VEC, 16, true>(a, stream);
+        if (H < 8) return launch_lsh<T, VEC, 8, false>(a, stream);
+        if (H < 16) return launch_lsh<T, VEC, 16, false>(a, stream);
+        return launch_lsh<T, VEC, 32, false>(a, stream);
+    }
 }
 
 template <typename T>
@@ -161,12 +551,14 @@ int lsh_hash_typed(int64_t N, int64_t F, int bits, const void *X, const void *W,
     constexpr int WIDE = 16 / sizeof(T);  // elements per 16-byte access
     const bool wide = (F % WIDE == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0);
     const int vec = wide ? WIDE : 1;
-    const int max_slab = kLshMaxSlab * 4 / (int)sizeof(T);
+    // single precision with 16-byte rows: whole rows of up to 512 bytes per pass
+    const int max_slab = sizeof(T) == sizeof(float) ? (wide ? kLshMfmaSlab : kLshMaxSlab) : kLshMaxSlab / 2;
     int slab = (int)(F < max_slab ? F : max_slab);
     slab -= slab % vec;
     a.slab = slab;
     const int slab_v = slab / vec;
     a.stride_v = slab_v | 1;
+    a.wstride = ((slab / 4) | 1) * 4;  // odd in 16-byte units: 16 planes read without bank conflicts
     a.magic = slab_v > 1 ? (uint32_t)((1ull << 32) / (uint32_t)slab_v) + 1u : 0u;  // 0: divide directly
     if (wide) return dispatch_lsh<T, WIDE>(a, stream);
     return dispatch_lsh<T, 1>(a, stream);

@@ -376,13 +376,15 @@ std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, 
     ok(cgnn_lsh_scan((int)bits, buckets.data_ptr<int32_t>(), prefix.data_ptr<int32_t>(), workspace[2].data_ptr(),
                      (size_t)workspace[2].numel(), stream),
        "lsh_scan");
-    // One scalar read, only when assignments are refreshed (cluster_kernel.cu:146-147).
-    const int active = prefix.select(0, n - 1).item<int>();
-    Tensor counts = torch::zeros({active + 1}, buckets.options());
+    // The number of active buckets is at most min(N, 2^bits): the last step runs on a
+    // buffer of that bound, so the device never waits for the host; the one scalar read
+    // of a refresh (cluster_kernel.cu:146-147) comes last and only trims the view.
+    Tensor counts = torch::zeros({std::min<int64_t>(N, n) + 1}, buckets.options());
     ok(cgnn_lsh_finish(N, (int)bits, raw.data_ptr<int32_t>(), buckets.data_ptr<int32_t>(), prefix.data_ptr<int32_t>(),
                        ids.data_ptr<int64_t>(), counts.data_ptr<int32_t>(), stream),
        "lsh_finish");
-    return {ids, counts, (int64_t)active};
+    const int active = prefix.select(0, n - 1).item<int>();
+    return {ids, counts.narrow(0, 0, active + 1), (int64_t)active};
 }
 
 // cluster_forward (src/runtime/csrc/cluster/cluster.cpp:12-30): int32 ids and the
