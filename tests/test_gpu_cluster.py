@@ -70,6 +70,44 @@ def test_assign_mean_reconstruct(dtype, width, n, bits):
             assert np.array_equal(rg[small], want_rg[small])
 
 
+@pytest.mark.parametrize("width,bits", [
+    (4, 3), (16, 16), (20, 9), (48, 17), (64, 30), (84, 12), (100, 16), (100, 24), (104, 16), (112, 7),
+    (124, 16), (128, 16), (128, 30), (132, 16), (256, 16), (300, 21), (512, 8), (37, 16), (130, 19)])
+def test_assign_shapes(width, bits):
+    """Ids and counts over the widths that select the different projection kernels
+    (whole-row tiles with 1..32 packs per row, padded and unpadded LDS strides, several
+    passes per tile, unaligned widths) and both plane-group counts, on enough rows
+    (100k + a partial tile) that every persistent wave walks several tiles."""
+    n = 100_003
+    rng = np.random.default_rng(width * 100 + bits)
+    x = rng.standard_normal((n, width)).astype(np.float32)
+    w = rng.standard_normal((width, bits)).astype(np.float32)
+    want_ids, want_counts, want_active = oracle.assign(x, w, bits)
+    ids, counts, active = abi.lsh_assign(_t(x), _t(w), bits)
+    torch.cuda.synchronize()
+    assert active == want_active
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert np.array_equal(counts.cpu().numpy(), want_counts)
+
+
+def test_assign_denormal_and_cancelling_projections():
+    """Projections that end exactly at zero, in the denormal range or one ulp from zero
+    decide bits by the last rounding: the chains must be fused multiply-adds."""
+    rng = np.random.default_rng(11)
+    n, width, bits = 4096, 8, 16
+    x = rng.standard_normal((n, width)).astype(np.float32)
+    w = rng.standard_normal((width, bits)).astype(np.float32)
+    x[:, 4:] = -x[:, :4]          # second half cancels the first when the planes repeat
+    w[4:, :8] = w[:4, :8]         # planes 0..7: exact cancellation -> h == 0 -> bit 0
+    w[4:, 8:] = np.nextafter(w[:4, 8:], np.float32(np.inf))  # planes 8..15: residue of one ulp
+    x[::3] *= np.float32(1e-22)   # products deep in the denormal range
+    want_ids, want_counts, want_active = oracle.assign(x, w, bits)
+    ids, counts, active = abi.lsh_assign(_t(x), _t(w), bits)
+    assert active == want_active
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert np.array_equal(counts.cpu().numpy(), want_counts)
+
+
 @pytest.mark.parametrize("bits", [0, 8, 24])
 def test_all_collide(bits):
     """Known answer of the reference's test: every row in one bucket -> count == [0, 513]."""
