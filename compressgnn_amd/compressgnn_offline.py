@@ -20,6 +20,7 @@ EXPORTS = [
     "cgnn_csr_transpose", "cgnn_hybird_partition", "cgnn_topo_partition", "cgnn_gen_degree",
     "cgnn_filter_csr", "cgnn_depth_filter_csr", "cgnn_gen_vertex_order_csr", "cgnn_gen_vertex_order_csc",
     "cgnn_compress_csr_batch", "cgnn_csr_hstack", "cgnn_csr_row_stats", "cgnn_gen_chung_lu", "cgnn_gen_copy_model",
+    "cgnn_add_self_loop_coo", "cgnn_gcn_norm_coo_compress", "cgnn_gen_edge_order",
 ]
 
 _NP_TYPES = {0: np.int64, 1: np.float32, 2: np.int32}
@@ -40,7 +41,8 @@ def lib():
             if name.startswith("cgnn_") and name not in (
                     "cgnn_arrays_count", "cgnn_arrays_type", "cgnn_arrays_size", "cgnn_arrays_data",
                     "cgnn_arrays_scalar", "cgnn_arrays_free", "cgnn_prep_last_error",
-                    "cgnn_get_norm_degree", "cgnn_gcn_norm_csr_compress", "cgnn_csr_row_stats"):
+                    "cgnn_get_norm_degree", "cgnn_gcn_norm_csr_compress", "cgnn_gcn_norm_coo_compress",
+                    "cgnn_csr_row_stats"):
                 getattr(L, name).restype = ctypes.c_void_p
         L.cgnn_arrays_free.argtypes = [ctypes.c_void_p]
         L.cgnn_arrays_count.argtypes = [ctypes.c_void_p]
@@ -217,6 +219,37 @@ def csr2coo(vlist, elist):
     vlist, elist = _i64(vlist), _i64(elist)
     src = np.repeat(np.arange(len(vlist) - 1, dtype=np.int64), np.diff(vlist))
     return src, elist.copy()
+
+
+def add_self_loop_coo(src, dst, vertex_cnt):
+    src, dst = _i64(src), _i64(dst)
+    (s, d), _ = _take(lib().cgnn_add_self_loop_coo(ctypes.c_int64(len(src)), _p(src), _p(dst),
+                                                   ctypes.c_int64(vertex_cnt)))
+    return s, d
+
+
+def gcn_norm_coo_compress(src, dst, norm_degree, vertex_cnt, rule_cnt):
+    src, dst, d = _i64(src), _i64(dst), _f32(norm_degree)
+    w = np.empty(len(src), dtype=np.float32)
+    if lib().cgnn_gcn_norm_coo_compress(ctypes.c_int64(len(src)), _p(src), _p(dst), _p(d),
+                                        ctypes.c_int64(vertex_cnt), ctypes.c_int64(rule_cnt), _p(w)):
+        raise RuntimeError(_err())
+    return w
+
+
+def gen_edge_order(src, dst, vertex_cnt, rule_cnt):
+    """(phase of every edge int32[E], number of phases)."""
+    src, dst = _i64(src), _i64(dst)
+    (order,), (phases,) = _take(lib().cgnn_gen_edge_order(ctypes.c_int64(len(src)), _p(src), _p(dst),
+                                                          ctypes.c_int64(vertex_cnt), ctypes.c_int64(rule_cnt)), 1)
+    return order, phases
+
+
+def gen_mask_edge(src, dst, vertex_cnt, rule_cnt):
+    """(bool mask [phases, E], phases): mask[k] selects the edges of phase k
+    (src/offline/csrc/gen_mask.h:86-108)."""
+    order, phases = gen_edge_order(src, dst, vertex_cnt, rule_cnt)
+    return order[None, :] == np.arange(phases, dtype=np.int32)[:, None], phases
 
 
 def csr_hstack(a0, a1, col_offset):

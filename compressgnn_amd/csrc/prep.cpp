@@ -14,6 +14,7 @@
 #include <cstdio>
 #include <cstring>
 #include <numeric>
+#include <stdexcept>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -765,6 +766,109 @@ cgnn_arrays *cgnn_gen_vertex_order_csc(int64_t V, int64_t R, const int64_t *vlis
         auto *out = new cgnn_arrays;
         out->add(std::move(order));
         out->scalars.push_back(depth);
+        return out;
+    });
+}
+
+cgnn_arrays *cgnn_add_self_loop_coo(int64_t E, const int64_t *src, const int64_t *dst, int64_t V) {
+    // Reference: src/offline/csrc/add_self_loop.h:55-107.  Edges are grouped by ascending
+    // source; (v, v) is placed behind v's targets below v unless it is already there.
+    // Edges whose source does not come up in that order are left out, as there.
+    if (E < 0 || V < 0 || (E > 0 && (!src || !dst))) {
+        set_error("add_self_loop_coo: bad arguments");
+        return nullptr;
+    }
+    return guarded([&] {
+        std::vector<i64> ns, nd;
+        ns.reserve((size_t)(E + V));
+        nd.reserve((size_t)(E + V));
+        i64 e = 0;
+        auto keep = [&] {
+            ns.push_back(src[e]);
+            nd.push_back(dst[e]);
+            ++e;
+        };
+        for (i64 v = 0; v < V; ++v) {
+            while (e < E && src[e] == v && dst[e] < v) keep();
+            if (e < E && src[e] == v && dst[e] == v) {
+                keep();
+            } else {
+                ns.push_back(v);
+                nd.push_back(v);
+            }
+            while (e < E && src[e] == v) keep();
+        }
+        auto *out = new cgnn_arrays;
+        out->add(std::move(ns));
+        out->add(std::move(nd));
+        return out;
+    });
+}
+
+int cgnn_gcn_norm_coo_compress(int64_t E, const int64_t *src, const int64_t *dst, const float *d, int64_t V,
+                               int64_t R, float *weight) {
+    // Reference: src/offline/csrc/norm.h:129-166.
+    if (E < 0 || V < 0 || R < 0 || (E > 0 && (!src || !dst || !weight)) || (V > 0 && !d)) {
+        set_error("gcn_norm_coo_compress: bad arguments");
+        return 1;
+    }
+    for (i64 e = 0; e < E; ++e) {
+        const i64 s = src[e], t = dst[e];
+        if (s < 0 || t < 0 || s >= V + R || t >= V + R) {
+            set_error("gcn_norm_coo_compress: edge %lld out of range", (long long)e);
+            return 1;
+        }
+        if (s < V) weight[e] = t < V ? d[s] * d[t] : d[s];
+        else weight[e] = t < V ? d[t] : 1.0f;
+    }
+    return 0;
+}
+
+cgnn_arrays *cgnn_gen_edge_order(int64_t E, const int64_t *src, const int64_t *dst, int64_t V, int64_t R) {
+    // Reference: src/offline/csrc/gen_mask.h:10-84.  Phase 0 holds every edge that leaves a
+    // vertex.  An edge that leaves a rule is due in the first phase after all rule->rule
+    // edges into that rule have been delivered; a rule that only vertices feed is complete
+    // after phase 0.  A phase is formed from the state at its start.
+    if (E < 0 || V < 0 || R < 0 || (E > 0 && (!src || !dst))) {
+        set_error("gen_edge_order: bad arguments");
+        return nullptr;
+    }
+    return guarded([&] {
+        std::vector<int32_t> order((size_t)E, -1);
+        std::vector<i64> waiting((size_t)R, 0);  // undelivered rule->rule edges into each rule
+        std::vector<i64> open;                   // edges that leave a rule, in input order
+        for (i64 e = 0; e < E; ++e) {
+            if (src[e] < 0 || dst[e] < 0 || src[e] >= V + R || dst[e] >= V + R)
+                throw std::runtime_error("gen_edge_order: edge out of range");
+            if (src[e] < V) {
+                order[e] = 0;
+            } else {
+                open.push_back(e);
+                if (dst[e] >= V) ++waiting[dst[e] - V];
+            }
+        }
+        int phases = 1;
+        std::vector<i64> later, delivered;
+        while (!open.empty()) {
+            later.clear();
+            delivered.clear();
+            for (i64 e : open) {
+                if (waiting[src[e] - V] == 0) {
+                    order[e] = phases;
+                    if (dst[e] >= V) delivered.push_back(dst[e] - V);
+                } else {
+                    later.push_back(e);
+                }
+            }
+            if (later.size() == open.size())
+                throw std::runtime_error("gen_edge_order: the rule graph has a cycle");
+            for (i64 r : delivered) --waiting[r];
+            open.swap(later);
+            ++phases;
+        }
+        auto *out = new cgnn_arrays;
+        out->add(std::move(order));
+        out->scalars.push_back(phases);
         return out;
     });
 }

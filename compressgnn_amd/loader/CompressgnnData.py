@@ -1,12 +1,14 @@
 """CompressgnnData: builds the compressed, normalised, partitioned graph from raw
 arrays.  Same constructor, fields, to() and __repr__ as the reference's
-loader/CompressgnnData.py:60-201 (graph_type="csr" branch)."""
+loader/CompressgnnData.py:60-201: graph_type="csr" yields a CompressGraph, graph_type="coo"
+per-phase edge lists and weights."""
 import _paths  # noqa: F401
 import numpy as np
 import torch
 
-from compressgnn_offline import (add_self_loop_csr, csr_transpose, depth_filter_csr, filter_csr,
-                                 gcn_norm_csr_compress, gen_vertex_order_csc, get_norm_degree)
+from compressgnn_offline import (add_self_loop_coo, add_self_loop_csr, coo2csr, csr2coo, csr_transpose,
+                                 depth_filter_csr, filter_csr, gcn_norm_coo_compress, gcn_norm_csr_compress,
+                                 gen_mask_edge, gen_vertex_order_csc, get_norm_degree)
 from compress_graph import CompressGraph
 from compression_backend import compress_graph_csr, resolve_backend
 
@@ -87,8 +89,36 @@ class CompressgnnData():
             colptr, row, value = csr_transpose(new_vlist, new_elist, edge_weight, total)
             self.edge_index = CompressGraph(colptr, row, value, self.vertex_cnt)
         elif self.graph_type == "coo":
-            raise NotImplementedError(
-                'graph_type="coo" (multi-phase scatter propagation) is not part of this build; use graph_type="csr"')
+            # reference loader/CompressgnnData.py:86-139: edges sorted by source
+            src = np.asarray(edge_index[0]).astype(np.int64)
+            dst = np.asarray(edge_index[1]).astype(np.int64)
+            if add_self_loop:
+                src, dst = add_self_loop_coo(src, dst, self.vertex_cnt)
+            if normalize:
+                norm_degree = get_norm_degree(dst, self.vertex_cnt)
+            vlist, elist = coo2csr(src, dst, self.vertex_cnt)
+            new_vlist, new_elist, new_vertex_cnt, new_rule_cnt = compress(
+                vlist, elist, threshold, max_depth, min_edge, min_pair_frequency,
+                self.compression_backend, compression_threads, compression_rounds, verbose)
+            self.vertex_cnt = new_vertex_cnt
+            self.rule_cnt = new_rule_cnt
+            self.edge_cnt = new_elist.shape[0]
+            src, dst = csr2coo(new_vlist, new_elist)
+            if normalize:
+                edge_weight = gcn_norm_coo_compress(src, dst, norm_degree, self.vertex_cnt, self.rule_cnt)
+            else:
+                edge_weight = np.ones(self.edge_cnt, dtype=np.float32)
+            edge_mask, step = gen_mask_edge(src, dst, self.vertex_cnt, self.rule_cnt)
+            if verbose:
+                print("step:{}".format(step))
+            self.step = step
+            pairs = torch.from_numpy(np.vstack((src, dst)))
+            weights = torch.from_numpy(edge_weight)
+            self.edge_index, self.edge_weight = [], []
+            for i in range(step):
+                mask = torch.from_numpy(edge_mask[i])
+                self.edge_index.append(torch.stack((pairs[0][mask], pairs[1][mask]), 0))
+                self.edge_weight.append(weights[mask])
         else:
             raise ValueError('graph_type must be "coo" or "csr"')
 
@@ -102,5 +132,10 @@ class CompressgnnData():
         self.train_mask = self.train_mask.to(device)
         self.vaild_mask = self.vaild_mask.to(device)
         self.test_mask = self.test_mask.to(device)
-        self.edge_index = self.edge_index.to(device)
+        if self.graph_type == "coo":
+            for i in range(self.step):
+                self.edge_index[i] = self.edge_index[i].to(device)
+                self.edge_weight[i] = self.edge_weight[i].to(device)
+        else:
+            self.edge_index = self.edge_index.to(device)
         return self

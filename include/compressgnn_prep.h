@@ -44,6 +44,22 @@ int cgnn_get_norm_degree(int64_t E, const int64_t *dst, int64_t V, float *out);
 int cgnn_gcn_norm_csr_compress(int64_t V, int64_t R, const int64_t *vlist, const int64_t *elist,
                                const float *norm_degree, float *weight);
 
+/* add_self_loop_coo (src/offline/csrc/add_self_loop.h:55-107): edges grouped by ascending
+ * source, targets ascending within a source; (v, v) is inserted behind v's targets below
+ * v unless present.  -> [src, dst] */
+cgnn_arrays *cgnn_add_self_loop_coo(int64_t E, const int64_t *src, const int64_t *dst, int64_t V);
+
+/* gcn_norm_coo_compress (norm.h:129-166): the edge weights of gcn_norm_csr_compress for
+ * an edge list (src -> dst) over V vertices followed by R rules. */
+int cgnn_gcn_norm_coo_compress(int64_t E, const int64_t *src, const int64_t *dst,
+                               const float *norm_degree, int64_t V, int64_t R, float *weight);
+
+/* gen_edge_order (src/offline/csrc/gen_mask.h:10-84), from which gen_mask_edge
+ * (gen_mask.h:86-108) forms its phase masks: phase 0 = edges that leave a vertex, phase
+ * k >= 1 = edges that leave a rule all of whose rule inputs arrived in phases < k.
+ * -> [order (int32, E)]; scalar: number of phases. */
+cgnn_arrays *cgnn_gen_edge_order(int64_t E, const int64_t *src, const int64_t *dst, int64_t V, int64_t R);
+
 /* CSR -> CSC of a rows x cols matrix: entries ordered by column, then by row, ties in
  * original order (the order torch_sparse's SparseTensor.csc() yields, which
  * loader/CompressgnnData.py:180 and layer/CompressgnnSPMM.py:68-70 rely on).

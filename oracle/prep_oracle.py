@@ -127,3 +127,72 @@ def expand(vlist, elist, node, V):
             assert np.all(children < child), "rule graph must be acyclic (children < rule)"
             stack.extend(reversed([int(c) for c in children]))
     return out
+
+
+def add_self_loop_coo(src, dst, vertex_cnt):
+    """src/offline/csrc/add_self_loop.h:55-107 (edges grouped by ascending source, targets
+    ascending within a source)."""
+    ns, nd = [], []
+    e, E = 0, len(src)
+    for v in range(vertex_cnt):
+        mine = []
+        while e < E and src[e] == v:
+            mine.append(int(dst[e]))
+            e += 1
+        below = [t for t in mine if t < v]
+        rest = mine[len(below):]
+        if not rest or rest[0] != v:
+            rest = [v] + rest
+        for t in below + rest:
+            ns.append(v)
+            nd.append(t)
+    return np.array(ns, np.int64), np.array(nd, np.int64)
+
+
+def gcn_norm_coo_compress(src, dst, d, V, R):
+    """src/offline/csrc/norm.h:129-166."""
+    w = np.empty(len(src), np.float32)
+    for e, (s, t) in enumerate(zip(src, dst)):
+        if s < V:
+            w[e] = np.float32(d[s] * d[t]) if t < V else d[s]
+        else:
+            w[e] = d[t] if t < V else np.float32(1)
+    return w
+
+
+def gen_edge_order(src, dst, V, R):
+    """src/offline/csrc/gen_mask.h:10-84: (phase of every edge, number of phases)."""
+    E = len(src)
+    order = np.full(E, -1, np.int32)
+    pending = np.zeros(R, np.int64)
+    for e in range(E):
+        if dst[e] >= V:
+            pending[dst[e] - V] += 1
+    for e in range(E):
+        if src[e] < V:
+            order[e] = 0
+            if dst[e] >= V:
+                pending[dst[e] - V] -= 1
+    step = 1
+    while (order < 0).any():
+        arrived = np.zeros(R, np.int64)
+        for e in range(E):
+            if src[e] >= V and order[e] < 0 and pending[src[e] - V] == 0:
+                order[e] = step
+                if dst[e] >= V and pending[dst[e] - V] > 0:
+                    arrived[dst[e] - V] += 1
+        pending -= arrived
+        step += 1
+    return order, step
+
+
+def coo_propagate(x, phases, weights, V, R):
+    """layer/CompressgnnPropagation.py:68-83 with KPropagate.message (layer/KPropagate.py:30-31)
+    and a sequential scatter-add in edge order: out[(V+R) x F] starts at zero, phase 0
+    gathers from x, later phases from out; returns out[:V]."""
+    out = np.zeros((V + R, x.shape[1]), x.dtype)
+    for k, (edges, w) in enumerate(zip(phases, weights)):
+        feat = x if k == 0 else out
+        msg = feat[edges[0]] if w is None else (w.reshape(-1, 1) * feat[edges[0]]).astype(x.dtype)
+        np.add.at(out, edges[1], msg)
+    return out[:V]

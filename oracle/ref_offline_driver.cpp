@@ -28,4 +28,8 @@ PYBIND11_MODULE(compressgnn_offline_ref, m) {
     m.def("hybird_partition", &hybird_partition);
     m.def("topo_partition", &topo_partition);
     m.def("gen_degree", &gen_degree);
+    m.def("add_self_loop_coo", &add_self_loop_coo);
+    m.def("gcn_norm_coo_compress", &gcn_norm_coo_compress);
+    m.def("gen_edge_order", &gen_edge_order);
+    m.def("gen_mask_edge", &gen_mask_edge);
 }

@@ -180,6 +180,29 @@ def make_offline():
                                 [lv[0] for lv in levels], [lv[1] for lv in levels])
         out.update({pre + "vertex_degree": np.asarray(vd), pre + "rule_degree": np.asarray(rd)})
     out["n_rule_graphs"] = np.array(len(graphs))
+    # edge-list (COO) forms: weights and phase order of the compressed graphs above, and
+    # self loops on plain sorted edge lists.  (The reference's add_self_loop_coo reads one
+    # element past its inputs; the arrays passed are views with a -1 behind the last edge.)
+    for i in range(len(graphs)):
+        pre = "r%d_" % i
+        V, R = int(out[pre + "V"]), int(out[pre + "R"])
+        src, dst = off.csr2coo(out[pre + "vlist"], out[pre + "elist"])
+        out[pre + "coo_weight"] = np.asarray(off.gcn_norm_coo_compress(src, dst, out[pre + "d"], V, R))
+        order, phases = off.gen_edge_order(src, dst, V, R)
+        out.update({pre + "edge_order": np.asarray(order), pre + "edge_phases": np.array(phases)})
+        mask, phases2 = off.gen_mask_edge(src, dst, V, R)
+        assert phases2 == phases and np.array_equal(np.asarray(mask), np.asarray(order)[None, :] == np.arange(phases)[:, None])
+    for i, (V, deg) in enumerate([(1, 0), (9, 2), (40, 4), (33, 6)]):
+        rows = [sorted(set(rng.integers(0, V, size=int(rng.integers(0, deg + 1))).tolist())) for _ in range(V)]
+        src = np.full(sum(len(r) for r in rows) + 1, -1, np.int64)
+        dst = src.copy()
+        src[:-1] = [v for v, r in enumerate(rows) for _ in r]
+        dst[:-1] = [c for r in rows for c in r]
+        s, d = off.add_self_loop_coo(src[:-1], dst[:-1], V)
+        pre = "c%d_" % i
+        out.update({pre + "V": np.array(V), pre + "src": src[:-1].copy(), pre + "dst": dst[:-1].copy(),
+                    pre + "sl_src": np.asarray(s), pre + "sl_dst": np.asarray(d)})
+    out["n_coo"] = np.array(4)
     np.savez_compressed(os.path.join(HERE, "offline_golden.npz"), **out)
 
 

@@ -97,9 +97,9 @@ def test_csc_is_the_stable_transpose():
 
 
 def test_unsupported_paths_fail_loudly():
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):
         CompressgnnData(np.zeros((2, 1)), (np.array([0, 1]), np.array([1, 0])), np.zeros(2), np.ones(2, bool),
-                        np.ones(2, bool), np.ones(2, bool), graph_type="coo")
+                        np.ones(2, bool), np.ones(2, bool), graph_type="ell")
     with pytest.raises(ValueError):
         CompressgnnData(np.zeros((2, 1)), (np.array([0, 1, 2]), np.array([1, 0])), np.zeros(2), np.ones(2, bool),
                         np.ones(2, bool), np.ones(2, bool), graph_type="csr", compression_backend="tpu")
@@ -123,3 +123,34 @@ def test_backend_resolution():
         dispatch.compress_graph_csr(np.array([0, 0]), np.array([], np.int64), 2)
     with pytest.raises(ValueError):
         dispatch.compress_graph_csr(np.array([0, 0]), np.array([], np.int64), 16, threads=0)
+
+
+def test_coo_phases_cover_the_compressed_graph():
+    """graph_type="coo": the phases partition the compressed edge list, phase 0 holds the
+    edges that leave vertices, and summing the phases in order (the oracle's sequential
+    scatter) reproduces the uncompressed normalised product."""
+    import compressgnn_offline as off
+    import prep_oracle
+    V = 2708
+    vl, el = off.gen_chung_lu(V, 10500, 2.5, 11)
+    src, dst = off.csr2coo(vl, el)
+    x = np.random.default_rng(2).standard_normal((V, 8)).astype(np.float32)
+    m = np.ones(V, bool)
+    data = CompressgnnData(x, (src, dst), np.zeros(V, np.int64), m, m, m, graph_type="coo",
+                           min_pair_frequency=3, threshold=0)
+    same = CompressgnnData(x, (vl, el), np.zeros(V, np.int64), m, m, m, graph_type="csr",
+                           min_pair_frequency=3, threshold=0)
+    assert (data.vertex_cnt, data.rule_cnt, data.edge_cnt) == (same.vertex_cnt, same.rule_cnt, same.edge_cnt)
+    assert data.rule_cnt > 0 and data.step == len(data.edge_index) == len(data.edge_weight) >= 2
+    assert sum(e.size(1) for e in data.edge_index) == data.edge_cnt
+    assert bool((data.edge_index[0][0] < V).all())
+    for e in data.edge_index[1:]:
+        assert bool((e[0] >= V).all())
+    out = prep_oracle.coo_propagate(x, [e.numpy() for e in data.edge_index], [w.numpy() for w in data.edge_weight],
+                                    data.vertex_cnt, data.rule_cnt)
+    s2, d2 = off.add_self_loop_coo(src, dst, V)
+    nd = off.get_norm_degree(d2, V).astype(np.float64)
+    want = np.zeros((V, 8))
+    np.add.at(want, d2, (nd[s2] * nd[d2])[:, None] * x[s2])
+    np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-5)
+    assert "coo" in repr(data) and data.to("cpu") is data

@@ -39,6 +39,34 @@ def test_self_loop_and_norm_degree_golden():
         assert eq(prep_oracle.get_norm_degree(se, len(v) - 1), nd)
 
 
+def test_edge_list_routines_golden():
+    """add_self_loop_coo, gcn_norm_coo_compress and the phase order of gen_edge_order /
+    gen_mask_edge against the compiled reference's outputs."""
+    for i in range(int(GOLD["n_coo"])):
+        p = "c%d_" % i
+        V = int(GOLD[p + "V"])
+        s, d = off.add_self_loop_coo(GOLD[p + "src"], GOLD[p + "dst"], V)
+        assert eq(s, GOLD[p + "sl_src"]) and eq(d, GOLD[p + "sl_dst"])
+        os_, od = prep_oracle.add_self_loop_coo(GOLD[p + "src"], GOLD[p + "dst"], V)
+        assert eq(os_, s) and eq(od, d)
+    for i in range(int(GOLD["n_rule_graphs"])):
+        p = "r%d_" % i
+        V, R = int(GOLD[p + "V"]), int(GOLD[p + "R"])
+        src, dst = off.csr2coo(GOLD[p + "vlist"], GOLD[p + "elist"])
+        w = off.gcn_norm_coo_compress(src, dst, GOLD[p + "d"], V, R)
+        assert w.dtype == np.float32 and eq(w, GOLD[p + "coo_weight"]) and eq(w, GOLD[p + "weight"])
+        assert eq(prep_oracle.gcn_norm_coo_compress(src, dst, GOLD[p + "d"], V, R), w)
+        order, phases = off.gen_edge_order(src, dst, V, R)
+        assert phases == int(GOLD[p + "edge_phases"]) and order.dtype == np.int32 and eq(order, GOLD[p + "edge_order"])
+        o2, p2 = prep_oracle.gen_edge_order(src, dst, V, R)
+        assert p2 == phases and eq(o2, order)
+        mask, p3 = off.gen_mask_edge(src, dst, V, R)
+        assert p3 == phases and mask.dtype == bool and mask.shape == (phases, len(src))
+        assert eq(mask.argmax(0), order) and int(mask.sum()) == len(src)
+    with pytest.raises(RuntimeError):
+        off.gen_edge_order(np.array([2, 3]), np.array([3, 2]), 2, 2)  # two rules feeding each other
+
+
 @pytest.mark.parametrize("i", range(int(GOLD["n_rule_graphs"])))
 def test_compressed_graph_routines_golden(i):
     p = "r%d_" % i
