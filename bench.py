@@ -16,6 +16,8 @@ resident in HBM.  Prints ONE JSON line:
   detail       per-stage times, plain-CSR comparison, cluster + reconstruct times (C3)
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cluster] [--skip-cpu]
+       python bench.py --c4 [--c4-vertices N]   (the large end-to-end configuration only:
+                                                 minutes of host-side graph preparation)
 """
 import argparse
 import json
@@ -292,6 +294,104 @@ def cpu_cluster_baseline(x, planes, detail, sample=200000):
         reconstruct_ms=(t3 - t2) * 1e3, reconstruct_backward_ms=(t5 - t4) * 1e3, mean_backward_ms=(t6 - t5) * 1e3)
 
 
+C4_VERTICES, C4_AVG_DEGREE, C4_F, C4_HIDDEN, C4_CLASSES, C4_H = 18_500_000, 16.1, 64, 64, 16, 16
+
+
+def bench_c4(torch, vertices, epochs, refresh_interval):
+    """C4: one training epoch of a 2-layer GCN whose layers are propagate -> cluster ->
+    Linear on the representatives -> reconstruct(bias) (the layer of the reference's
+    model/compressgnn/gcn.py:27-34), ReLU between the layers, log-softmax + NLL over all
+    vertices, Adam; on a copy-model graph (same generator and seed as C1, average
+    out-degree 16.1) with N(0,1) features and uniform random labels."""
+    import torch.nn.functional as Fn
+    import compressgnn_offline as off
+    from CompressgnnCluster import Compressgnn_Cluster
+    from CompressgnnData import CompressgnnData
+    from CompressgnnReconstruct import Compressgnn_Reconstruct
+    from KPropagate import KPropagate
+
+    dev = torch.device("cuda:0")
+    times = {}
+    t0 = time.time()
+    v, e = off.gen_copy_model(vertices, C4_AVG_DEGREE, C1_COPY_PROB, C1_SEED)
+    times["generate_s"] = time.time() - t0
+    log("[bench] C4 graph generated: V=%d E=%d (%.1fs)" % (vertices, len(e), times["generate_s"]))
+    t0 = time.time()
+    mask = np.ones(1, dtype=bool)  # masks are not used: the loss runs over all vertices
+    data = CompressgnnData(np.zeros((vertices, 1), np.float32), (v, e), np.zeros(1, np.int64), mask, mask, mask,
+                           add_self_loop=True, normalize=True, graph_type="csr")
+    times["compress_and_partition_s"] = time.time() - t0
+    edges = int(len(e))
+    del v, e
+    graph = data.edge_index
+    log("[bench] C4 compressed: rules=%d compressed edges=%d levels=%d (%.1fs)"
+        % (data.rule_cnt, data.edge_cnt, graph.step, times["compress_and_partition_s"]))
+    t0 = time.time()
+    graph.to(dev)
+    graph.plan()
+    torch.cuda.synchronize()
+    times["to_device_and_plan_s"] = time.time() - t0
+    log("[bench] C4 plan on device (%.1fs)" % times["to_device_and_plan_s"])
+
+    class Layer(torch.nn.Module):
+        def __init__(self, fin, fout):
+            super().__init__()
+            self.lin = torch.nn.Linear(fin, fout, bias=True)
+            self.P = KPropagate()
+            self.cluster = Compressgnn_Cluster(in_feature=fin, param_H=C4_H, training=True, cache=True,
+                                               refresh_interval=refresh_interval)
+            self.reconstruct = Compressgnn_Reconstruct()
+
+        def forward(self, x, epoch):
+            x = self.P(x=x, edge_index=graph, edge_weight=None, vertex_cnt=data.vertex_cnt, rule_cnt=data.rule_cnt)
+            reps, index = self.cluster(x, epoch=epoch)
+            return self.reconstruct(Fn.linear(reps, self.lin.weight, None), index, bias=self.lin.bias)
+
+    torch.manual_seed(0)
+    layers = torch.nn.ModuleList([Layer(C4_F, C4_HIDDEN), Layer(C4_HIDDEN, C4_CLASSES)]).to(dev)
+    opt = torch.optim.Adam(layers.parameters(), lr=0.01)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    x = torch.randn(vertices, C4_F, device=dev, generator=gen)
+    y = torch.randint(0, C4_CLASSES, (vertices,), device=dev, generator=gen)
+    torch.cuda.reset_peak_memory_stats()
+
+    def epoch(k):
+        opt.zero_grad(set_to_none=True)
+        h = layers[0](x, k).relu()
+        out = Fn.log_softmax(layers[1](h, k), dim=1)
+        loss = Fn.nll_loss(out, y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    losses, ms = [], []
+    for k in range(epochs + 1):  # epoch 0 is the warm-up (first-use allocations, plan caches)
+        torch.cuda.synchronize()
+        t0 = time.time()
+        loss = epoch(k)
+        torch.cuda.synchronize()
+        ms.append((time.time() - t0) * 1e3)
+        losses.append(float(loss.detach()))
+        log("[bench] C4 epoch %d: %.1f ms, loss %.4f" % (k, ms[-1], losses[-1]))
+    timed = ms[1:]
+    refreshed = [layers[0].cluster.refresh_count, layers[1].cluster.refresh_count]
+    return {
+        "metric": "gcn_2layer_epoch_ms_C4", "value": float(np.mean(timed)), "unit": "ms", "n_gpus": 1,
+        "steps": epochs, "warmup": 1, "ms_per_step": float(np.mean(timed)), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "C4: 2-layer GCN training epoch (propagate -> cluster -> linear -> reconstruct per "
+                               "layer), copy-model graph %d vertices / %d directed edges, F=%d hidden=%d classes=%d "
+                               "param_H=%d refresh_interval=%d" % (vertices, edges, C4_F, C4_HIDDEN, C4_CLASSES,
+                                                                   C4_H, refresh_interval),
+                   "rules": int(data.rule_cnt), "compressed_edges": int(data.edge_cnt), "levels": int(graph.step)},
+        "detail": {"epoch_ms": ms, "loss": losses, "cluster_refreshes": refreshed,
+                   "peak_hbm_bytes": int(torch.cuda.max_memory_allocated()),
+                   "active_clusters": [int(layers[0].cluster.active_bucket), int(layers[1].cluster.active_bucket)],
+                   "host_seconds": times},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,6 +401,11 @@ def main():
     ap.add_argument("--skip-cluster", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--sweep", action="store_true", help="also time F in {16, 64, 256, 512} (C2)")
+    ap.add_argument("--c4", action="store_true",
+                    help="run only the large end-to-end configuration (2-layer GCN epoch) and print its line")
+    ap.add_argument("--c4-vertices", type=int, default=C4_VERTICES)
+    ap.add_argument("--c4-epochs", type=int, default=3)
+    ap.add_argument("--c4-refresh-interval", type=int, default=1)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path uses no "
@@ -310,6 +415,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     import compressgnn_runtime as rt
     from CompressgnnSPMM import compress_spmm  # noqa: F401  (the layer path uses the same plan)
+    if args.c4:
+        print(json.dumps(bench_c4(torch, args.c4_vertices, args.c4_epochs, args.c4_refresh_interval)))
+        return
 
     F = args.features
     dev = torch.device("cuda:0")
