@@ -215,7 +215,6 @@ def bench_cluster(torch, steps, detail):
     planes = torch.randn(C3_F, C3_H, device=dev, generator=gen)
     weight = (torch.rand(C3_OUT, C3_F, device=dev, generator=gen) * 2 - 1) / (C3_F ** 0.5)
     bias = (torch.rand(C3_OUT, device=dev, generator=gen) * 2 - 1) / (C3_F ** 0.5)
-    ws = rt.cluster_workspace(x, C3_H)
 
     def timed(fn, reps=steps):
         fn()
@@ -229,9 +228,9 @@ def bench_cluster(torch, steps, detail):
         return a.elapsed_time(b) / reps, out
 
     N, F, Fo = C3_NODES, C3_F, C3_OUT
-    t_assign, (ids, counts, active) = timed(lambda: rt.cluster_assign(x, planes, C3_H, ws))
+    # one refresh: hash codes, group them by a sort -> ids, counts and member lists
+    t_assign, (ids, counts, active, members) = timed(lambda: rt.cluster_assign_members(x, planes, C3_H))
     groups = active + 1
-    t_members, members = timed(lambda: rt.cluster_members(ids, groups))
     t_mean, reps = timed(lambda: rt.cluster_mean(x, ids, counts, members))
     t_linear, hidden = timed(lambda: torch.nn.functional.linear(reps, weight))
     t_recon, out = timed(lambda: rt.cluster_reconstruct(hidden, ids, bias, True, members))
@@ -242,8 +241,7 @@ def bench_cluster(torch, steps, detail):
     gb = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
     C = groups
     ops = {
-        "assign": dict(ms=t_assign, bytes=4 * N * F + 4 * F * C3_H + 8 * N),
-        "members": dict(ms=t_members, bytes=8 * N + 8 * N + 4 * C),
+        "assign": dict(ms=t_assign, bytes=4 * N * F + 4 * F * C3_H + 8 * N + 8 * N + 4 * C),
         "mean": dict(ms=t_mean, bytes=4 * N * F + 8 * N + 4 * C * F),
         "reconstruct": dict(ms=t_recon, bytes=4 * C * Fo + 8 * N + 4 * Fo + 4 * N * Fo),
         "reconstruct_backward": dict(ms=t_recon_bwd, bytes=2 * 4 * N * Fo + 8 * N + 4 * C * Fo),
@@ -253,7 +251,7 @@ def bench_cluster(torch, steps, detail):
         v["GBps"] = gb(v["bytes"], v["ms"])
         v["frac_of_hbm_peak"] = v["GBps"] / HBM_PEAK_GBPS
     reuse = t_mean + t_linear + t_recon + t_recon_bwd + t_linear_bwd + t_mean_bwd
-    refresh = reuse + t_assign + t_members
+    refresh = reuse + t_assign
     detail["cluster_reconstruct_C3"] = dict(
         nodes=N, in_features=F, bits=C3_H, out_features=Fo, active_clusters=int(active), ops=ops,
         linear_ms=t_linear, linear_backward_ms=t_linear_bwd,
@@ -360,7 +358,7 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
         opt.zero_grad(set_to_none=True)
         h = layers[0](x, k).relu()
         out = Fn.log_softmax(layers[1](h, k), dim=1)
-        loss = Fn.nll_loss(out, y)
+        loss = -out.gather(1, y.unsqueeze(1)).mean()  # NLL over all vertices
         loss.backward()
         opt.step()
         return loss

@@ -20,6 +20,7 @@ EXPORTS = [
     "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
     "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_hash", "cgnn_lsh_scan", "cgnn_lsh_finish",
+    "cgnn_lsh_group_workspace_bytes", "cgnn_lsh_group",
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
     "cgnn_cluster_mean_workspace_bytes", "cgnn_cluster_mean", "cgnn_cluster_mean_backward",
     "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_copy_bytes",
@@ -46,7 +47,7 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.cgnn_last_error.restype = ctypes.c_char_p
         L.cgnn_version.restype = ctypes.c_char_p
-        for name in ("cgnn_spmm_workspace_bytes", "cgnn_lsh_scan_workspace_bytes",
+        for name in ("cgnn_spmm_workspace_bytes", "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_group_workspace_bytes",
                      "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
         _lib = L
@@ -176,6 +177,30 @@ def lsh_assign(x, planes, bits):
     counts = torch.zeros(active + 1, dtype=torch.int32, device=dev)
     check(L.cgnn_lsh_finish(i64(N), bits, ptr(raw), ptr(bucket_count), ptr(prefix), ptr(ids), ptr(counts), st))
     return ids, counts, active
+
+
+def lsh_assign_grouped(x, planes, bits):
+    """(ids, counts, active, (offsets, perm, sorted_id)) through cgnn_lsh_hash without
+    counters and cgnn_lsh_group (sort by code); one host read of the group count."""
+    N, F = x.shape
+    dev = x.device
+    L = lib()
+    cap = min(N, 1 << bits)
+    raw = torch.empty(N, dtype=torch.int32, device=dev)
+    ids = torch.empty(N, dtype=torch.int64, device=dev)
+    perm = torch.empty(N, dtype=torch.int32, device=dev)
+    sorted_id = torch.empty(N, dtype=torch.int32, device=dev)
+    offsets = torch.empty(cap + 2, dtype=torch.int32, device=dev)
+    counts = torch.zeros(cap + 1, dtype=torch.int32, device=dev)
+    active = torch.zeros(1, dtype=torch.int32, device=dev)
+    st = stream_of(x)
+    check(L.cgnn_lsh_hash(i64(N), i64(F), bits, dtype_code(x.dtype), ptr(x), ptr(planes), ptr(raw), None, st))
+    need = L.cgnn_lsh_group_workspace_bytes(i64(N), bits)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    check(L.cgnn_lsh_group(i64(N), bits, ptr(raw), ptr(ids), ptr(offsets), ptr(perm), ptr(sorted_id), ptr(counts),
+                           ptr(active), ptr(ws), ctypes.c_size_t(need), st))
+    n = int(active.item())
+    return ids, counts[:n + 1], n, (offsets[:n + 2], perm, sorted_id)
 
 
 def cluster_members(ids, groups):

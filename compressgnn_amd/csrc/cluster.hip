@@ -34,6 +34,77 @@ constexpr int kLshMaxSlab = 32;  // columns staged per pass (floats): 9 KB of LD
 __device__ __forceinline__ float fused_mul_add(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fused_mul_add(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+// Histogram update of one wave.  Feature rows of a graph are far from uniform: a few
+// codes can hold most rows, and atomics on one counter serialise in the memory system.
+// The wave therefore keeps kHeld (code, count) pairs in wave-uniform registers across its
+// calls.  Per call: lanes whose code is held are added to that pair; then, up to kHeld
+// times, the first lane still uncounted leads, every lane with its code is counted with
+// it, and the pair replaces a held pair that saw no lane in this call (whose count is sent
+// with one atomic), or is sent at once if every held pair was used; lanes left over count
+// themselves.  A code that keeps turning up stays held until flush(), so a dominant code
+// costs one atomic per wave instead of one per row.
+constexpr int kHeld = 4;
+
+// Where the (code, count) pairs of a wave go: the global counters.
+struct GlobalSink {
+    int32_t *bucket_count;
+    __device__ __forceinline__ void operator()(int code, int n) const { atomicAdd(bucket_count + code, n); }
+};
+
+struct WaveCodeCounter {
+    int code_[kHeld] = {-1, -1, -1, -1};
+    int count_[kHeld] = {0, 0, 0, 0};
+    int next_ = 0;
+
+    template <typename Sink>
+    __device__ __forceinline__ void flush(const Sink &sink, int lane) {
+#pragma unroll
+        for (int k = 0; k < kHeld; ++k) {
+            if (count_[k] > 0 && lane == 0) sink(code_[k], count_[k]);
+            count_[k] = 0;
+        }
+    }
+    template <typename Sink>
+    __device__ __forceinline__ void add(const Sink &sink, int code, bool valid, int lane) {
+        unsigned long long todo = __ballot(valid);
+        unsigned used = 0;
+#pragma unroll
+        for (int k = 0; k < kHeld; ++k) {
+            const unsigned long long m = __ballot(valid && code == code_[k]);  // codes are >= 0
+            count_[k] += __popcll(m);
+            todo &= ~m;
+            if (m != 0) used |= 1u << k;
+        }
+        for (int round = 0; round < kHeld && todo != 0; ++round) {
+            const int leader = __ffsll(todo) - 1;
+            const int lead = __builtin_amdgcn_readlane(code, leader);
+            const unsigned long long same = __ballot(valid && code == lead);
+            const int n = __popcll(same);
+            todo &= ~same;
+            int victim = -1;
+#pragma unroll
+            for (int j = 0; j < kHeld; ++j) {
+                const int k = (next_ + j) % kHeld;
+                if (victim < 0 && !((used >> k) & 1u)) victim = k;
+            }
+            if (victim < 0) {
+                if (lane == leader) sink(lead, n);
+                continue;
+            }
+#pragma unroll
+            for (int k = 0; k < kHeld; ++k)
+                if (k == victim) {
+                    if (count_[k] > 0 && lane == 0) sink(code_[k], count_[k]);
+                    code_[k] = lead;
+                    count_[k] = n;
+                }
+            used |= 1u << victim;
+            next_ = (victim + 1) % kHeld;
+        }
+        if ((todo >> lane) & 1) sink(code, 1);
+    }
+};
+
 template <typename T>
 struct LshArgs {
     const T *__restrict__ X;
@@ -100,14 +171,16 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_kernel(LshArgs<T> a) {
             }
         }
     }
-    if (lane < rows_here) {
-        int code = 0;
+    int code = 0;
 #pragma unroll
-        for (int j = 0; j < HB; ++j)
-            if (j < H) code = (code << 1) | (acc[j] > T(0) ? 1 : 0);
-        a.raw_code[row0 + lane] = code;
-        atomicAdd(a.bucket_count + code, 1);
-    }
+    for (int j = 0; j < HB; ++j)
+        if (j < H) code = (code << 1) | (acc[j] > T(0) ? 1 : 0);
+    if (lane < rows_here) a.raw_code[row0 + lane] = code;
+    if (a.bucket_count == nullptr) return;
+    WaveCodeCounter counter;
+    const GlobalSink sink{a.bucket_count};
+    counter.add(sink, code, lane < rows_here, lane);
+    counter.flush(sink, lane);
 }
 
 // Single precision runs the same chains on the matrix unit.  v_mfma_f32_16x16x1_4b_f32
@@ -221,6 +294,8 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_mfma_kernel(LshArgs<float> 
     // The wave walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...; while it multiplies
     // one pass out of LDS, the next pass (of this tile or of the next one) is in flight.
     const int myv = 4 * (lane >> 4) + (lane & 3);
+    WaveCodeCounter counter;
+    const GlobalSink sink{a.bucket_count};
     if (slabs == 1) stage_planes(0);  // same planes for every tile; ordered before the first pass's reads
     fetch(blockIdx.x, 0);
     for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
@@ -277,15 +352,14 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_mfma_kernel(LshArgs<float> 
             }
         }
         const int64_t row = t * kLshRows + lane;
-        if (row < a.N) {
-            const int shift = 16 * ((lane & 15) >> 2);
-            uint32_t mask = (uint32_t)(sel[0] >> shift) & 0xffffu;  // bit j = (h_j > 0)
-            if (NG == 2) mask |= ((uint32_t)(sel[NG - 1] >> shift) & 0xffffu) << 16;
-            const int code = (int)(__brev(mask) >> (32 - H));  // plane 0 is the top bit
-            a.raw_code[row] = code;
-            atomicAdd(a.bucket_count + code, 1);
-        }
+        const int shift = 16 * ((lane & 15) >> 2);
+        uint32_t mask = (uint32_t)(sel[0] >> shift) & 0xffffu;  // bit j = (h_j > 0)
+        if (NG == 2) mask |= ((uint32_t)(sel[NG - 1] >> shift) & 0xffffu) << 16;
+        const int code = (int)(__brev(mask) >> (32 - H));  // plane 0 is the top bit
+        if (row < a.N) a.raw_code[row] = code;
+        if (a.bucket_count != nullptr) counter.add(sink, code, row < a.N, lane);
     }
+    counter.flush(sink, lane);
 }
 
 // Whole rows per pass (F <= 128, 16-byte packs): the 64 rows of a tile are one contiguous
@@ -315,6 +389,7 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
     const lsh_f4_t *X4 = reinterpret_cast<const lsh_f4_t *>(a.X);
     const int64_t first = (int64_t)blockIdx.x * waves + wave;
     const int64_t step = (int64_t)gridDim.x * waves;
+    const GlobalSink sink{a.bucket_count};
 
     for (int e = threadIdx.x; e < a.F * 16 * NG; e += blockDim.x) {  // planes as [plane][k]
         const int kk = e / (16 * NG), j = e % (16 * NG);
@@ -362,6 +437,7 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
                     acc[g] = __builtin_amdgcn_mfma_f32_16x16x1f32(x[i][k], w[g][i][k], acc[g], 0, 0, 0);
     };
 
+    WaveCodeCounter counter;
     int pending_code = 0;
     int64_t pending_row = -1;
     if (first < tiles) fetch(first);
@@ -373,10 +449,8 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
             if (u < ks_v) tile[p + (padded ? (int)__umulhi((uint32_t)p, a.magic) : 0)] = xr[u];
         }
         wave_lds_sync();
-        if (pending_row >= 0 && pending_row < a.N) {
-            a.raw_code[pending_row] = pending_code;
-            atomicAdd(a.bucket_count + pending_code, 1);
-        }
+        if (pending_row >= 0 && pending_row < a.N) a.raw_code[pending_row] = pending_code;
+        if (a.bucket_count != nullptr) counter.add(sink, pending_code, pending_row >= 0 && pending_row < a.N, lane);
         if (t + step < tiles) fetch(t + step);
 
         // eight column packs at a time: all sixteen LDS reads are issued before the first
@@ -405,17 +479,16 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
         pending_code = (int)(__brev(mask) >> (32 - H));  // plane 0 is the top bit
         pending_row = t * kLshRows + lane;
     }
-    if (pending_row >= 0 && pending_row < a.N) {
-        a.raw_code[pending_row] = pending_code;
-        atomicAdd(a.bucket_count + pending_code, 1);
-    }
+    if (pending_row >= 0 && pending_row < a.N) a.raw_code[pending_row] = pending_code;
+    if (a.bucket_count != nullptr) counter.add(sink, pending_code, pending_row >= 0 && pending_row < a.N, lane);
+    counter.flush(sink, lane);
 }
 
 // bits == 0 or F == 0: every projection is empty, code 0.
 __global__ void lsh_trivial_kernel(int32_t *raw_code, int32_t *bucket_count, int64_t N) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < N) raw_code[i] = 0;
-    if (i == 0) bucket_count[0] = (int32_t)N;
+    if (i == 0 && bucket_count != nullptr) bucket_count[0] = (int32_t)N;
 }
 
 __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
@@ -478,10 +551,11 @@ int launch_lsh_flat(const LshArgs<float> &a, hipStream_t stream) {
     const size_t tile_bytes = (size_t)kLshRows * a.stride_v * sizeof(lsh_f4_t);
     const size_t plane_bytes = (size_t)a.wstride * 16 * NG * sizeof(float);
     // as many waves as fit beside one copy of the planes; two per SIMD at most (registers)
-    int waves = (int)((kLdsPerCu - plane_bytes) / tile_bytes);
+    const size_t fixed_bytes = plane_bytes;
+    int waves = (int)((kLdsPerCu - fixed_bytes) / tile_bytes);
     waves = waves < 1 ? 1 : (waves > kLshFlatMaxWaves ? kLshFlatMaxWaves : waves);
     auto kernel = lsh_hash_mfma_flat_kernel<NG, XP>;
-    size_t lds = plane_bytes + waves * tile_bytes;
+    size_t lds = fixed_bytes + waves * tile_bytes;
     if (lds > kLdsDefaultLimit) {
         static bool allowed = false, refused = false;  // per kernel instantiation
         if (!allowed && !refused) {
@@ -494,9 +568,9 @@ int launch_lsh_flat(const LshArgs<float> &a, hipStream_t stream) {
             }
         }
         if (!allowed) {
-            waves = (int)((kLdsDefaultLimit - plane_bytes) / tile_bytes);
+            waves = (int)((kLdsDefaultLimit - fixed_bytes) / tile_bytes);
             waves = waves < 1 ? 1 : waves;
-            lds = plane_bytes + waves * tile_bytes;
+            lds = fixed_bytes + waves * tile_bytes;
         }
     }
     return launch_lsh_persistent(kernel, waves, lds, a, stream);
@@ -809,6 +883,19 @@ cgnn_csr members_csr(int64_t N, int64_t groups, const int32_t *offsets, const in
 }
 
 }  // namespace
+// out[i] = #{j <= i : in[j] != 0} over n int32 entries; scratch of occupancy_scan_bytes(n).
+size_t occupancy_scan_bytes(int64_t n) { return align_up((size_t)ceil_div(n < 1 ? 1 : n, kScanTile) * sizeof(int32_t), 256); }
+
+int occupancy_scan(const int32_t *in, int64_t n, int32_t *out, void *scratch, hipStream_t stream) {
+    if (n <= 0) return CGNN_OK;
+    const int64_t tiles = ceil_div(n, kScanTile);
+    int32_t *totals = static_cast<int32_t *>(scratch);
+    hipLaunchKernelGGL(scan_tile_totals_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, in, n, totals);
+    hipLaunchKernelGGL(scan_totals_kernel, dim3(1), dim3(kBlock), 0, stream, totals, tiles);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, in, n, totals, out);
+    return check_launch("occupancy_scan");
+}
+
 }  // namespace cgnn
 
 using namespace cgnn;
@@ -820,9 +907,8 @@ extern "C" int cgnn_lsh_hash(int64_t N, int64_t F, int bits, int dtype, const vo
     CGNN_REQUIRE(N >= 0 && F >= 0, "cgnn_lsh_hash: negative size");
     CGNN_REQUIRE(N < INT32_MAX, "cgnn_lsh_hash: row count exceeds the int32 bucket counters");
     CGNN_REQUIRE(F < (1 << 24), "cgnn_lsh_hash: feature width too large");
-    CGNN_REQUIRE(bucket_count != nullptr, "cgnn_lsh_hash: bucket_count is null");
     CGNN_REQUIRE(N == 0 || raw_code != nullptr, "cgnn_lsh_hash: raw_code is null");
-    rc = fill_i32(bucket_count, (int64_t)1 << bits, 0, stream);
+    if (bucket_count != nullptr) rc = fill_i32(bucket_count, (int64_t)1 << bits, 0, stream);
     if (rc != CGNN_OK || N == 0) return rc;
     if (bits == 0 || F == 0) {
         hipLaunchKernelGGL(lsh_trivial_kernel, dim3((unsigned)ceil_div(N, kBlock)), dim3(kBlock), 0,

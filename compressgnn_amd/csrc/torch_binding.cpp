@@ -344,7 +344,51 @@ std::vector<Tensor> cluster_workspace(Tensor input, int64_t bits) {
             torch::empty({(int64_t)cgnn_lsh_scan_workspace_bytes((int)bits)}, input.options().dtype(torch::kUInt8))};
 }
 
-// cluster_assign_cuda (cluster_kernel.cu:118-153).
+// Assignment and member lists of one refresh: ids [N] int64 (1-based), counts
+// [active+1] int32 (entry 0 = 0), active, and the member lists (offsets [active+2], perm
+// [N], sorted_id [N]).  The codes are grouped by a stable sort instead of bucket counters,
+// so the result is the same as cluster_assign_cuda's (cluster_kernel.cu:118-153) whatever
+// the distribution of the codes, and the member lists come with it.  The number of groups
+// is at most min(N, 2^bits): every kernel runs on buffers of that bound, so the device
+// never waits for the host; the one scalar read of a refresh (cluster_kernel.cu:146-147)
+// comes last and only trims the views.
+std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(Tensor input, Tensor planes,
+                                                                                int64_t bits) {
+    check_float(input);
+    check_float(planes);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    const int n = bucket_size(bits);
+    TORCH_CHECK(planes.device() == input.device() && planes.scalar_type() == input.scalar_type() &&
+                    planes.size(0) == input.size(1) && planes.size(1) == bits,
+                "Hash plane shape/device/dtype mismatch");
+    TORCH_CHECK(input.size(0) < INT_MAX, "Node count exceeds int32 capacity");
+    const int64_t N = input.size(0);
+    auto ints = input.options().dtype(torch::kInt32);
+    Tensor ids = torch::empty({N}, input.options().dtype(torch::kInt64));
+    Tensor perm = torch::empty({N}, ints), sorted_id = torch::empty({N}, ints);
+    if (N == 0)
+        return {ids, torch::zeros({1}, ints), 0, {torch::zeros({2}, ints), perm, sorted_id}};
+    const int64_t cap = std::min<int64_t>(N, n);
+    Tensor raw = torch::empty({N}, ints);
+    Tensor offsets = torch::empty({cap + 2}, ints), counts = torch::empty({cap + 1}, ints);
+    Tensor active_dev = torch::empty({1}, ints);
+    auto stream = current_stream(input);
+    ok(cgnn_lsh_hash(N, input.size(1), (int)bits, dtype_code(input), input.data_ptr(), planes.data_ptr(),
+                     raw.data_ptr<int32_t>(), nullptr, stream),
+       "lsh_hash");
+    const size_t bytes = cgnn_lsh_group_workspace_bytes(N, (int)bits);
+    Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, input.options().dtype(torch::kUInt8));
+    ok(cgnn_lsh_group(N, (int)bits, raw.data_ptr<int32_t>(), ids.data_ptr<int64_t>(), offsets.data_ptr<int32_t>(),
+                      perm.data_ptr<int32_t>(), sorted_id.data_ptr<int32_t>(), counts.data_ptr<int32_t>(),
+                      active_dev.data_ptr<int32_t>(), ws.data_ptr(), bytes, stream),
+       "lsh_group");
+    const int active = active_dev.item<int>();
+    return {ids, counts.narrow(0, 0, active + 1), (int64_t)active,
+            {offsets.narrow(0, 0, active + 2), perm, sorted_id}};
+}
+
+// cluster_assign_cuda (cluster_kernel.cu:118-153).  The workspace of cluster_workspace is
+// checked as there; the grouping itself no longer needs bucket counters.
 std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, int64_t bits,
                                                    std::vector<Tensor> workspace) {
     check_float(input);
@@ -364,27 +408,8 @@ std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, 
                     workspace[0].numel() == n && workspace[1].numel() == n &&
                     workspace[2].scalar_type() == torch::kUInt8 && (size_t)workspace[2].numel() >= scan_bytes,
                 "Workspace dtype/capacity mismatch");
-    const int64_t N = input.size(0);
-    Tensor ids = torch::empty({N}, input.options().dtype(torch::kInt64));
-    if (N == 0) return {ids, torch::zeros({1}, workspace[0].options()), 0};
-    auto stream = current_stream(input);
-    Tensor raw = torch::empty({N}, workspace[0].options());
-    Tensor buckets = workspace[0], prefix = workspace[1];
-    ok(cgnn_lsh_hash(N, input.size(1), (int)bits, dtype_code(input), input.data_ptr(), planes.data_ptr(),
-                     raw.data_ptr<int32_t>(), buckets.data_ptr<int32_t>(), stream),
-       "lsh_hash");
-    ok(cgnn_lsh_scan((int)bits, buckets.data_ptr<int32_t>(), prefix.data_ptr<int32_t>(), workspace[2].data_ptr(),
-                     (size_t)workspace[2].numel(), stream),
-       "lsh_scan");
-    // The number of active buckets is at most min(N, 2^bits): the last step runs on a
-    // buffer of that bound, so the device never waits for the host; the one scalar read
-    // of a refresh (cluster_kernel.cu:146-147) comes last and only trims the view.
-    Tensor counts = torch::zeros({std::min<int64_t>(N, n) + 1}, buckets.options());
-    ok(cgnn_lsh_finish(N, (int)bits, raw.data_ptr<int32_t>(), buckets.data_ptr<int32_t>(), prefix.data_ptr<int32_t>(),
-                       ids.data_ptr<int64_t>(), counts.data_ptr<int32_t>(), stream),
-       "lsh_finish");
-    const int active = prefix.select(0, n - 1).item<int>();
-    return {ids, counts.narrow(0, 0, active + 1), (int64_t)active};
+    auto grouped = cluster_assign_members(input, planes, bits);
+    return {std::get<0>(grouped), std::get<1>(grouped), std::get<2>(grouped)};
 }
 
 // cluster_forward (src/runtime/csrc/cluster/cluster.cpp:12-30): int32 ids and the
@@ -539,6 +564,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("cluster_forward", &cluster_forward, "CompressGNN cluster forward");
     m.def("cluster_workspace", &cluster_workspace);
     m.def("cluster_assign", &cluster_assign);
+    m.def("cluster_assign_members", &cluster_assign_members,
+          "(ids, counts, active, [offsets, perm, sorted_id]) of one assignment refresh");
     m.def("cluster_mean", &cluster_mean, py::arg("input"), py::arg("index"), py::arg("count"),
           py::arg("members") = py::none());
     m.def("cluster_mean_backward", &cluster_mean_backward, py::arg("grad"), py::arg("index"), py::arg("count"),

@@ -83,11 +83,14 @@ class _Mean(torch.autograd.Function):
 
 
 def _assign(input, planes, bits, workspace=None):
-    """reference layer/CompressgnnCluster.py:41-50 (GPU branch)"""
+    """reference layer/CompressgnnCluster.py:41-50 (GPU branch).  One call yields the
+    assignment and its member lists (the rows are grouped by a sort of their codes); the
+    lists are recorded for the index tensor.  The bucket workspace of the reference's
+    operator is not needed by this path."""
     with torch.no_grad():
-        if workspace is None:
-            workspace = _native.cluster_workspace(input.contiguous(), bits)
-        return _native.cluster_assign(input.contiguous(), planes.contiguous(), bits, workspace)
+        index, counts, active, members = _native.cluster_assign_members(input.contiguous(), planes.contiguous(), bits)
+        _remember(index, tuple(members))
+        return index, counts, active
 
 
 class Compressgnn_Cluster_Function(torch.autograd.Function):
@@ -197,7 +200,7 @@ class Compressgnn_Cluster(torch.nn.Module):
             self.set_epoch(epoch)
         if self.cache and self._epoch is None and (self.refresh_interval > 1 or self.refresh_policy == 'loss'):
             raise ValueError('Cross-epoch reuse requires set_epoch(epoch) or forward(epoch=epoch)')
-        # A workspace belongs to one device/stream; independent streams never share it.
+        # Assignments are kept per mode, device and stream.
         stream = torch.cuda.current_stream(input.device).cuda_stream if input.is_cuda else None
         slot = (self.training, input.device, stream)
         signature = (tuple(input.shape), input.dtype, cache_key, self.random_vectors.data_ptr(),
@@ -206,21 +209,14 @@ class Compressgnn_Cluster(torch.nn.Module):
         refresh = (not self.cache or force_refresh or self._epoch is None or state is None or
                    state['signature'] != signature or self._epoch - state['epoch'] >= self.current_interval)
         if refresh:
-            workspace = None
-            if input.is_cuda and input.size(0):
-                workspace_key = (input.device, stream, self.param_H)
-                if workspace_key not in self._workspaces:
-                    self._workspaces[workspace_key] = _native.cluster_workspace(input.contiguous(), self.param_H)
-                workspace = self._workspaces[workspace_key]
             if not input.size(0):
                 index = torch.empty(0, device=input.device, dtype=torch.int64)
                 counts = torch.zeros(1, device=input.device, dtype=torch.int32)
                 active = 0
             else:
-                index, counts, active = _assign(input, self.random_vectors, self.param_H, workspace)
-                # member lists of the new assignment, reused by every mean and
-                # reconstruct-gradient until the next refresh
-                _remember(index, _native.cluster_members(index, counts.numel()))
+                # the member lists of the new assignment come with it and are reused by
+                # every mean and reconstruct-gradient until the next refresh
+                index, counts, active = _assign(input, self.random_vectors, self.param_H)
             state = dict(index=index, counts=counts, active=active, signature=signature, epoch=self._epoch)
             if self.cache and self._epoch is not None:
                 self._states[slot] = state

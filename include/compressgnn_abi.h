@@ -119,6 +119,9 @@ size_t cgnn_lsh_scan_workspace_bytes(int bits);
 int cgnn_lsh_hash(int64_t N, int64_t F, int bits, int dtype, const void *X, const void *W,
                   int32_t *raw_code, int32_t *bucket_count, cgnn_stream_t stream);
 
+/* bucket_count may be NULL: then only raw_code is produced (cgnn_lsh_group derives the
+ * counts from the codes without any atomic update). */
+
 /* Step 2: prefix[b] = number of occupied buckets with index <= b (inclusive scan,
  * cluster_kernel.cu:143-145).  prefix[2^bits - 1] is the number of active buckets;
  * the caller reads it back (the one host synchronisation of cluster_kernel.cu:147). */
@@ -140,6 +143,19 @@ size_t cgnn_cluster_members_workspace_bytes(int64_t N, int64_t groups);
 int cgnn_cluster_members(int64_t N, int64_t groups, const int64_t *ids, int32_t *offsets,
                          int32_t *perm, int32_t *sorted_id, void *workspace,
                          size_t workspace_bytes, cgnn_stream_t stream);
+
+/* Steps 2 and 3 and the member lists in one, from the raw codes alone (no bucket
+ * counters): rows are sorted by code (stable), a run of equal codes is a group, and the
+ * 1-based id of a group is the rank of its code.  Produces what cgnn_lsh_scan +
+ * cgnn_lsh_finish + cgnn_cluster_members produce -- ids[N], counts[active+1] (entry 0 = 0),
+ * offsets[active+2], perm[N], sorted_id[N] -- and *active (device scalar) = number of
+ * groups.  counts needs room for min(N, 2^bits)+1 entries and offsets for one more; entries
+ * beyond active+1 (active+2) are left untouched.  Replaces cluster_kernel.cu:143-150 and
+ * the atomics of hash_ids (cluster_kernel.cu:41-59). */
+size_t cgnn_lsh_group_workspace_bytes(int64_t N, int bits);
+int cgnn_lsh_group(int64_t N, int bits, const int32_t *raw_code, int64_t *ids, int32_t *offsets,
+                   int32_t *perm, int32_t *sorted_id, int32_t *counts, int32_t *active,
+                   void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
 
 /* reps[g,:] = (sum over members i of group g, ascending i, of X[i,:]) / max(counts[g],1).
  * Replaces cluster_mean_cuda (cluster_kernel.cu:158-170). */

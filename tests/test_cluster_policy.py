@@ -36,6 +36,11 @@ class OracleNative:
         ids, counts, active = oracle.assign(x.detach().numpy(), planes.detach().numpy(), bits)
         return torch.from_numpy(ids), torch.from_numpy(counts), active
 
+    @classmethod
+    def cluster_assign_members(cls, x, planes, bits):
+        index, counts, active = cls.cluster_assign(x, planes, bits, None)
+        return index, counts, active, cls.cluster_members(index, active + 1)
+
     @staticmethod
     def cluster_members(index, groups):
         order = np.argsort(index.numpy(), kind="stable")

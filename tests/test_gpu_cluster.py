@@ -90,6 +90,39 @@ def test_assign_shapes(width, bits):
     assert np.array_equal(counts.cpu().numpy(), want_counts)
 
 
+@pytest.mark.parametrize("shape", ["uniform", "one_code", "few_codes", "relu"])
+@pytest.mark.parametrize("bits", [1, 8, 16, 23])
+def test_grouped_assign_matches_counter_path(shape, bits):
+    """cgnn_lsh_group (sort of the codes) against cgnn_lsh_hash/scan/finish (bucket
+    counters) + cgnn_cluster_members and against the oracle, on code distributions from
+    uniform to everything in one code: ids, counts, active and member lists are identical."""
+    rng = np.random.default_rng(bits * 7 + len(shape))
+    n, width = 70_001, 24
+    x = rng.standard_normal((n, width)).astype(np.float32)
+    if shape == "one_code":
+        x[:] = x[0]
+    elif shape == "few_codes":
+        x = x[rng.integers(0, 5, size=n) ** 2 % 7]
+    elif shape == "relu":
+        x = np.maximum(x - 1.0, 0).astype(np.float32)
+    w = rng.standard_normal((width, bits)).astype(np.float32)
+    want_ids, want_counts, want_active = oracle.assign(x, w, bits)
+    ids0, counts0, active0 = abi.lsh_assign(_t(x), _t(w), bits)
+    members0 = abi.cluster_members(ids0, active0 + 1)
+    ids, counts, active, members = abi.lsh_assign_grouped(_t(x), _t(w), bits)
+    torch.cuda.synchronize()
+    assert active == active0 == want_active
+    assert np.array_equal(ids.cpu().numpy(), want_ids) and torch.equal(ids, ids0)
+    assert np.array_equal(counts.cpu().numpy(), want_counts) and torch.equal(counts, counts0)
+    for got, ref in zip(members, members0):
+        assert got.dtype == ref.dtype and torch.equal(got, ref)
+
+
+def test_grouped_assign_empty():
+    ids, counts, active, members = abi.lsh_assign_grouped(torch.zeros(0, 8, device=DEV), torch.randn(8, 8, device=DEV), 8)
+    assert ids.numel() == 0 and active == 0 and counts.tolist() == [0] and members[0].tolist() == [0, 0]
+
+
 def test_assign_denormal_and_cancelling_projections():
     """Projections that end exactly at zero, in the denormal range or one ulp from zero
     decide bits by the last rounding: the chains must be fused multiply-adds."""
