@@ -192,15 +192,15 @@ def lsh_assign_grouped(x, planes, bits):
     sorted_id = torch.empty(N, dtype=torch.int32, device=dev)
     offsets = torch.empty(cap + 2, dtype=torch.int32, device=dev)
     counts = torch.zeros(cap + 1, dtype=torch.int32, device=dev)
-    active = torch.zeros(1, dtype=torch.int32, device=dev)
+    active = torch.zeros(2, dtype=torch.int32, device=dev)  # number of groups, largest group
     st = stream_of(x)
     check(L.cgnn_lsh_hash(i64(N), i64(F), bits, dtype_code(x.dtype), ptr(x), ptr(planes), ptr(raw), None, st))
     need = L.cgnn_lsh_group_workspace_bytes(i64(N), bits)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
     check(L.cgnn_lsh_group(i64(N), bits, ptr(raw), ptr(ids), ptr(offsets), ptr(perm), ptr(sorted_id), ptr(counts),
                            ptr(active), ptr(ws), ctypes.c_size_t(need), st))
-    n = int(active.item())
-    return ids, counts[:n + 1], n, (offsets[:n + 2], perm, sorted_id)
+    n, largest = (int(v) for v in active.cpu())
+    return ids, counts[:n + 1], n, (offsets[:n + 2], perm, sorted_id, largest)
 
 
 def cluster_members(ids, groups):
@@ -218,15 +218,15 @@ def cluster_members(ids, groups):
     return offsets, perm, sorted_id
 
 
-def cluster_mean(x, members, counts):
-    offsets, perm, sorted_id = members
+def cluster_mean(x, members, counts, max_members=0):
+    offsets, perm, sorted_id = members[:3]
     N, F = x.shape
     groups = counts.numel()
     L = lib()
     reps = torch.empty((groups, F), dtype=x.dtype, device=x.device)
     need = L.cgnn_cluster_mean_workspace_bytes(i64(N), i64(F), i64(groups), dtype_code(x.dtype))
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
-    check(L.cgnn_cluster_mean(i64(N), i64(F), i64(groups), dtype_code(x.dtype), ptr(x), ptr(offsets),
+    check(L.cgnn_cluster_mean(i64(N), i64(F), i64(groups), i64(max_members), dtype_code(x.dtype), ptr(x), ptr(offsets),
                               ptr(perm), ptr(sorted_id), ptr(counts), ptr(reps), ptr(ws),
                               ctypes.c_size_t(need), stream_of(x)))
     return reps
@@ -253,14 +253,14 @@ def reconstruct(reps, ids, bias=None, relu=False, members=None):
     return out
 
 
-def reconstruct_backward(grad, output, members, groups, relu=False):
-    offsets, perm, sorted_id = members
+def reconstruct_backward(grad, output, members, groups, relu=False, max_members=0):
+    offsets, perm, sorted_id = members[:3]
     N, F = grad.shape
     L = lib()
     reps_grad = torch.empty((groups, F), dtype=grad.dtype, device=grad.device)
     need = L.cgnn_cluster_mean_workspace_bytes(i64(N), i64(F), i64(groups), dtype_code(grad.dtype))
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=grad.device)
-    check(L.cgnn_reconstruct_backward(i64(N), i64(F), i64(groups), dtype_code(grad.dtype), ptr(grad),
+    check(L.cgnn_reconstruct_backward(i64(N), i64(F), i64(groups), i64(max_members), dtype_code(grad.dtype), ptr(grad),
                                       ptr(output), ptr(offsets), ptr(perm), ptr(sorted_id),
                                       ctypes.c_int(1 if relu else 0), ptr(reps_grad), ptr(ws),
                                       ctypes.c_size_t(need), stream_of(grad)))

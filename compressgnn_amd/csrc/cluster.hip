@@ -868,7 +868,7 @@ int check_bits(int bits) {
 size_t scan_tiles(int bits) { return (size_t)ceil_div((int64_t)1 << bits, kScanTile); }
 
 cgnn_csr members_csr(int64_t N, int64_t groups, const int32_t *offsets, const int32_t *perm,
-                     const int32_t *sorted_id) {
+                     const int32_t *sorted_id, int64_t max_members = 0) {
     cgnn_csr A{};
     A.rows = groups;
     A.cols = N;
@@ -877,7 +877,7 @@ cgnn_csr members_csr(int64_t N, int64_t groups, const int32_t *offsets, const in
     A.colidx = perm;
     A.rowidx = sorted_id;
     A.val = nullptr;
-    A.max_row_nnz = 0;
+    A.max_row_nnz = max_members > 0 && max_members < INT32_MAX ? (int32_t)max_members : 0;
     A.seg_nnz = 0;  // default run length: measured best for both cluster sums
     return A;
 }
@@ -978,7 +978,7 @@ static int divide_counts(void *reps, const int32_t *counts, int64_t groups, int6
     return check_launch("divide_counts");
 }
 
-extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype, const void *X,
+extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int64_t max_members, int dtype, const void *X,
                                  const int32_t *offsets, const int32_t *perm,
                                  const int32_t *sorted_id, const int32_t *counts, void *reps,
                                  void *workspace, size_t workspace_bytes, cgnn_stream_t stream) {
@@ -987,7 +987,7 @@ extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype
     if (F == 0) return CGNN_OK;
     CGNN_REQUIRE(offsets && counts && reps, "cgnn_cluster_mean: null array");
     CGNN_REQUIRE(N == 0 || (X && perm && sorted_id), "cgnn_cluster_mean: null array");
-    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id);
+    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id, max_members);
     int rc = spmm_members(&A, dtype, X, nullptr, reps, F, false, workspace, workspace_bytes, stream);
     if (rc != CGNN_OK) return rc;
     if (dtype == CGNN_F32) return divide_counts<float>(reps, counts, groups, F, stream);
@@ -1040,7 +1040,7 @@ extern "C" int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype,
     return fail(CGNN_EUNSUPPORTED, "cgnn_reconstruct: dtype must be f32 or f64");
 }
 
-extern "C" int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int dtype,
+extern "C" int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int64_t max_members, int dtype,
                                          const void *grad, const void *output,
                                          const int32_t *offsets, const int32_t *perm,
                                          const int32_t *sorted_id, int relu, void *reps_grad,
@@ -1052,7 +1052,7 @@ extern "C" int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, i
     CGNN_REQUIRE(offsets && reps_grad, "cgnn_reconstruct_backward: null array");
     CGNN_REQUIRE(N == 0 || (grad && perm && sorted_id), "cgnn_reconstruct_backward: null array");
     CGNN_REQUIRE(!relu || N == 0 || output, "cgnn_reconstruct_backward: relu needs the saved output");
-    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id);
+    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id, max_members);
     return spmm_members(&A, dtype, grad, output, reps_grad, F, relu != 0, workspace, workspace_bytes,
                         stream);
 }

@@ -48,7 +48,8 @@ __global__ void iota_kernel(int32_t *__restrict__ rows, int64_t N) {
 
 // head[p] = 1 where a run of equal codes starts.
 __global__ void group_heads_kernel(const int32_t *__restrict__ sorted_code, int64_t N,
-                                   int32_t *__restrict__ head) {
+                                   int32_t *__restrict__ head, int32_t *__restrict__ summary) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) summary[1] = 0;  // running maximum of the group sizes
     for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < N;
          p += (int64_t)gridDim.x * blockDim.x)
         head[p] = (p == 0 || sorted_code[p] != sorted_code[p - 1]) ? 1 : 0;
@@ -72,18 +73,26 @@ __global__ void group_finish_kernel(int64_t N, const int32_t *__restrict__ rank,
     }
 }
 
-__global__ void group_counts_kernel(const int32_t *__restrict__ offsets, const int32_t *__restrict__ active,
+// summary[0] = number of groups (set by group_finish_kernel), summary[1] = largest group.
+__global__ void group_counts_kernel(const int32_t *__restrict__ offsets, int32_t *__restrict__ summary,
                                     int32_t *__restrict__ counts, int64_t capacity) {
-    const int64_t groups = min((int64_t)*active, capacity) + 1;
+    const int64_t groups = min((int64_t)summary[0], capacity) + 1;
+    int largest = 0;
     for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups;
-         g += (int64_t)gridDim.x * blockDim.x)
-        counts[g] = g == 0 ? 0 : offsets[g + 1] - offsets[g];
+         g += (int64_t)gridDim.x * blockDim.x) {
+        const int c = g == 0 ? 0 : offsets[g + 1] - offsets[g];
+        counts[g] = c;
+        largest = max(largest, c);
+    }
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) largest = max(largest, __shfl_xor(largest, d, kWave));
+    if (threadIdx.x % kWave == 0 && largest > 0) atomicMax(summary + 1, largest);
 }
 
-__global__ void group_empty_kernel(int32_t *offsets, int32_t *counts, int32_t *active) {
+__global__ void group_empty_kernel(int32_t *offsets, int32_t *counts, int32_t *summary) {
     offsets[0] = offsets[1] = 0;
     counts[0] = 0;
-    *active = 0;
+    summary[0] = summary[1] = 0;
 }
 
 int key_bits(int64_t groups) {
@@ -125,13 +134,13 @@ extern "C" size_t cgnn_lsh_group_workspace_bytes(int64_t N, int bits) {
 }
 
 extern "C" int cgnn_lsh_group(int64_t N, int bits, const int32_t *raw_code, int64_t *ids, int32_t *offsets,
-                              int32_t *perm, int32_t *sorted_id, int32_t *counts, int32_t *active,
+                              int32_t *perm, int32_t *sorted_id, int32_t *counts, int32_t *summary,
                               void *workspace, size_t workspace_bytes, cgnn_stream_t stream) {
     CGNN_REQUIRE(N >= 0 && N < INT32_MAX, "cgnn_lsh_group: row count must be in [0, 2^31)");
     CGNN_REQUIRE(bits >= 0 && bits <= 30, "cgnn_lsh_group: bits must be in [0, 30]");
-    CGNN_REQUIRE(offsets && counts && active, "cgnn_lsh_group: null output");
+    CGNN_REQUIRE(offsets && counts && summary, "cgnn_lsh_group: null output");
     if (N == 0) {
-        hipLaunchKernelGGL(group_empty_kernel, dim3(1), dim3(1), 0, stream, offsets, counts, active);
+        hipLaunchKernelGGL(group_empty_kernel, dim3(1), dim3(1), 0, stream, offsets, counts, summary);
         return check_launch("lsh_group");
     }
     CGNN_REQUIRE(raw_code && ids && perm && sorted_id, "cgnn_lsh_group: null array");
@@ -154,15 +163,15 @@ extern "C" int cgnn_lsh_group(int64_t N, int bits, const int32_t *raw_code, int6
         set_error("cgnn_lsh_group: radix sort: %s", hipGetErrorString(e));
         return CGNN_ELAUNCH;
     }
-    hipLaunchKernelGGL(group_heads_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, sorted_code, N, head);
+    hipLaunchKernelGGL(group_heads_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, sorted_code, N, head, summary);
     int rc = occupancy_scan(head, N, sorted_id, scan_scratch, stream);
     if (rc != CGNN_OK) return rc;
     hipLaunchKernelGGL(group_finish_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, N, sorted_id, head,
-                       perm, ids, offsets, active);
+                       perm, ids, offsets, summary);
     const int64_t capacity = std::min<int64_t>(N, (int64_t)1 << bits);
     int64_t cblocks = ceil_div(capacity + 1, kBlock);
     if (cblocks > 4096) cblocks = 4096;
-    hipLaunchKernelGGL(group_counts_kernel, dim3((unsigned)cblocks), dim3(kBlock), 0, stream, offsets, active,
+    hipLaunchKernelGGL(group_counts_kernel, dim3((unsigned)cblocks), dim3(kBlock), 0, stream, offsets, summary,
                        counts, capacity);
     return check_launch("lsh_group");
 }

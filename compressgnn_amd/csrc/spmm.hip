@@ -16,8 +16,12 @@
 //     of any length cost the same).  Rows of at most seg_nnz entries always lie inside
 //     one run and are summed exactly as in the row schedule.  Longer rows are cut at
 //     multiples of seg_nnz: the part that continues into the next run is stored as a
-//     carry row and added by spmm_fixup_kernel, which walks the carries of one row in
-//     ascending run order.  No atomics anywhere, so results are reproducible run to run.
+//     carry row.  The carries of one row are consecutive; spmm_carry_reduce_kernel sums
+//     them 64 at a time, level by level (a row with a million entries is not walked by
+//     one lane group), and spmm_fixup_kernel adds what is left, in ascending order.
+//     Every output element receives its additions in a fixed order (where an atomic add
+//     is used it is the only addition to that element), so results are reproducible run
+//     to run.
 //
 // Modes: VAL (stored values), UNIT (all values 1), RELU_MASK (unit values, gathered
 // rows zeroed where a second matrix is <= 0), DUAL (columns below `split` gather from
@@ -56,6 +60,8 @@ struct SpmmArgs {
     T *Y;
     int32_t *carry_row;  // [nseg] row a run carries into, or -1
     T *carry;            // [nseg x F]
+    int32_t *carry_row_out;  // spmm_carry_reduce_kernel: the next, 32 times shorter level
+    T *carry_out;
     int64_t F;
     int32_t rows;
     int32_t nnz;
@@ -310,13 +316,112 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = continues ? cur : -1;
 }
 
+// One level of the carry reduction.  Carries (row, vector) with equal rows are adjacent;
+// -1 marks a run that carries nothing.  A lane group takes kCarryFan consecutive carries:
+// a row whose carries all lie inside the chunk is finished here (Y += their sum, nobody
+// else touches that row); the part of a row that reaches the chunk from before goes to
+// slot 2*chunk of the next level, the part of a row that goes on behind the chunk to slot
+// 2*chunk+1 (a row that covers the whole chunk fills slot 2*chunk and puts zeros in the
+// other), so that equal rows are adjacent again on the next level.
+constexpr int kCarryFan = 64;
+constexpr int kReduceBatch = 16;  // carry rows in flight per lane group
+constexpr int kFixBatch = 8;
+
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kBlock) void spmm_carry_reduce_kernel(SpmmArgs<T> a) {
+    constexpr int GPB = kBlock / LPR;
+    const int sub = threadIdx.x % LPR;
+    const int chunk = blockIdx.x * GPB + threadIdx.x / LPR;
+    const int s0 = chunk * kCarryFan;
+    if (s0 >= a.nseg) return;
+    const int s1 = min(s0 + kCarryFan, a.nseg);
+    const int before = s0 > 0 ? a.carry_row[s0 - 1] : -1;
+    const int after = s1 < a.nseg ? a.carry_row[s1] : -1;
+    // the rows of the chunk: every lane of the group reads all of them (same addresses,
+    // one round trip), so no lane has to wait for another
+    int rr[kCarryFan];
+    if (s1 - s0 == kCarryFan) {
+        const int4 *p = reinterpret_cast<const int4 *>(a.carry_row + s0);  // s0 is a multiple of 64
+#pragma unroll
+        for (int q = 0; q < kCarryFan / 4; ++q) {
+            const int4 v = p[q];
+            rr[4 * q] = v.x, rr[4 * q + 1] = v.y, rr[4 * q + 2] = v.z, rr[4 * q + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < kCarryFan; ++u) rr[u] = s0 + u < s1 ? a.carry_row[s0 + u] : -1;
+    }
+    int any = -1;
+#pragma unroll
+    for (int u = 0; u < kCarryFan; ++u) any = max(any, rr[u]);
+    if (any < 0) {  // nothing is carried through this chunk
+        if (sub == 0) a.carry_row_out[2 * chunk] = a.carry_row_out[2 * chunk + 1] = -1;
+        return;
+    }
+    int head_row = -1, tail_row = -1;
+    T *slot0 = a.carry_out + (int64_t)(2 * chunk) * a.F;
+    T *slot1 = slot0 + a.F;
+    for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC) {
+        Pack<T, VEC> acc, zero;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc.v[i] = zero.v[i] = T(0);
+        int cur = -1;
+        bool from_before = false;
+        auto close = [&](bool ends_here) {
+            if (cur < 0) return;
+            if (!from_before && ends_here) {
+                // The one addition to these elements in this launch sequence (the row's
+                // last run has stored its part already), so its result does not depend on
+                // timing; sent as an atomic only so that the lane need not wait for Y.
+                T *y = a.Y + (int64_t)cur * a.F + f;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) unsafeAtomicAdd(y + i, acc.v[i]);
+                return;
+            }
+            if (from_before) {
+                head_row = cur;
+                store_pack<T, VEC>(slot0 + f, acc);
+                if (!ends_here) {
+                    tail_row = cur;
+                    store_pack<T, VEC>(slot1 + f, zero);
+                }
+            } else {
+                tail_row = cur;
+                store_pack<T, VEC>(slot1 + f, acc);
+            }
+        };
+#pragma unroll
+        for (int b = 0; b < kCarryFan; b += kReduceBatch) {
+            Pack<T, VEC> c[kReduceBatch];
+#pragma unroll
+            for (int u = 0; u < kReduceBatch; ++u)
+                c[u] = rr[b + u] >= 0 ? load_pack<T, VEC>(a.carry + (int64_t)(s0 + b + u) * a.F + f) : zero;
+#pragma unroll
+            for (int u = 0; u < kReduceBatch; ++u) {
+                if (rr[b + u] != cur) {  // entries behind the end of the last chunk are -1
+                    close(true);
+                    cur = rr[b + u];
+                    acc = zero;
+                    from_before = (b + u == 0) && cur >= 0 && cur == before;
+                }
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
+            }
+        }
+        close(!(cur >= 0 && cur == after));
+    }
+    if (sub == 0) {
+        a.carry_row_out[2 * chunk] = head_row;
+        a.carry_row_out[2 * chunk + 1] = tail_row;
+    }
+}
+
 // Adds the carries of every row that straddles runs, in ascending run order, and
 // (when not accumulating) clears the rows that have no entries.  One thread looks at
 // one work item: item i < nseg is run i, which matters if it holds the first carry of
 // its row; item i < rows is row i, which matters if it is empty (the two sets of rows
 // are disjoint).  The items of a wave that matter are then dealt out to its lane groups
 // (LPR lanes across the features), kFixBatch carry rows in flight per group.
-constexpr int kFixBatch = 8;
 
 // Lane (within the wave) of the flagged item this lane's group should handle in the
 // round that starts at rank `base`, or -1.  Uniform control flow: every lane calls it.
@@ -443,7 +548,7 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
     return s;
 }
 
-enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2 };
+enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2, KIND_REDUCE = 3 };
 
 template <typename T, int VEC, int LPR, int TILES>
 int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int grid_y, hipStream_t stream) {
@@ -469,6 +574,10 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
             break;
         case KIND_FIXUP:
             hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, kBlock)), block, 0, stream, a);
+            break;
+        case KIND_REDUCE:  // items = chunks of kCarryFan carries, one lane group each
+            hipLaunchKernelGGL((spmm_carry_reduce_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, GPB)), block, 0,
+                               stream, a);
             break;
     }
     return check_launch("spmm launch");
@@ -554,7 +663,42 @@ SpmmArgs<T> make_args(const cgnn_csr *A, const void *X, const void *X1, int64_t 
     return a;
 }
 
-size_t carry_row_bytes(int64_t nseg) { return align_up((size_t)nseg * sizeof(int32_t), 256); }
+// Workspace of the nnz schedule: per level the rows of the carries, then the carries.
+// Level 0 has one carry per run; every further level has two per kCarryFan carries of the
+// one before; levels are added until at most kSerialCarries carries are left.
+constexpr int64_t kSerialCarries = 256;
+constexpr int kMaxCarryLevels = 8;
+
+struct CarryLevels {
+    int count = 0;
+    int64_t n[kMaxCarryLevels];
+    size_t row_off[kMaxCarryLevels], carry_off[kMaxCarryLevels];
+    size_t total = 0;
+};
+
+// Rows known to span fewer than kLongChain runs need no reduction levels: the fix-up
+// pass walks such chains directly.  max_row_nnz == 0 means unknown.
+constexpr int64_t kLongChain = 1024;
+
+bool wants_levels(const cgnn_csr *A, int seg) {
+    return A->max_row_nnz <= 0 || (int64_t)A->max_row_nnz > kLongChain * seg;
+}
+
+CarryLevels carry_levels(int64_t nseg, int64_t F, size_t elt, bool reduce) {
+    CarryLevels L;
+    int64_t n = nseg;
+    while (n > 0) {
+        const int k = L.count++;
+        L.n[k] = n;
+        L.row_off[k] = L.total;
+        L.total += align_up((size_t)n * sizeof(int32_t), 256);
+        L.carry_off[k] = L.total;
+        L.total += align_up((size_t)n * (size_t)F * elt, 256);
+        if (!reduce || n <= kSerialCarries || L.count == kMaxCarryLevels) break;
+        n = 2 * ceil_div(n, kCarryFan);
+    }
+    return L;
+}
 
 template <typename T>
 int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, const void *M, void *Y, int64_t F,
@@ -574,21 +718,39 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     if (A->nnz > 0 && A->rowidx == nullptr) return fail(CGNN_EINVAL, "spmm: nnz schedule needs rowidx");
     const int seg = seg_len(A);
     const int64_t nseg = ceil_div(A->nnz, seg);
-    const size_t need = carry_row_bytes(nseg) + (size_t)nseg * F * sizeof(T);
-    if (nseg > 0 && (ws == nullptr || ws_bytes < need)) {
-        set_error("spmm: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+    const CarryLevels levels = carry_levels(nseg, F, sizeof(T), wants_levels(A, seg));
+    if (nseg > 0 && (ws == nullptr || ws_bytes < levels.total)) {
+        set_error("spmm: workspace of %zu bytes needed, %zu given", levels.total, ws_bytes);
         return CGNN_EWORKSPACE;
     }
+    char *base = static_cast<char *>(ws);
+    auto level_rows = [&](int k) { return reinterpret_cast<int32_t *>(base + levels.row_off[k]); };
+    auto level_carries = [&](int k) { return reinterpret_cast<T *>(base + levels.carry_off[k]); };
     a.nseg = (int32_t)nseg;
     a.seg_nnz = seg;
-    a.carry_row = static_cast<int32_t *>(ws);
-    a.carry = reinterpret_cast<T *>(static_cast<char *>(ws) + carry_row_bytes(nseg));
-    Shape s = pick_shape<T>(F, X, Y, nseg > 0 ? a.carry : nullptr, mode == MODE_DUAL ? X1 : M);
+    a.carry_row = nseg > 0 ? level_rows(0) : nullptr;
+    a.carry = nseg > 0 ? level_carries(0) : nullptr;
+    Shape s = pick_shape<T>(F, X, Y, a.carry, mode == MODE_DUAL ? X1 : M);
     if (nseg > 0) {
         int rc = launch<T>(KIND_NNZ, mode, s, a, nseg, stream);
         if (rc != CGNN_OK) return rc;
     }
-    const int64_t items = accumulate ? nseg : (nseg > A->rows ? nseg : A->rows);
+    for (int k = 0; k + 1 < levels.count; ++k) {
+        a.nseg = (int32_t)levels.n[k];
+        a.carry_row = level_rows(k);
+        a.carry = level_carries(k);
+        a.carry_row_out = level_rows(k + 1);
+        a.carry_out = level_carries(k + 1);
+        int rc = launch<T>(KIND_REDUCE, mode, s, a, ceil_div(levels.n[k], kCarryFan), stream);
+        if (rc != CGNN_OK) return rc;
+    }
+    if (levels.count > 0) {
+        const int last = levels.count - 1;
+        a.nseg = (int32_t)levels.n[last];
+        a.carry_row = level_rows(last);
+        a.carry = level_carries(last);
+    }
+    const int64_t items = accumulate ? a.nseg : (a.nseg > A->rows ? a.nseg : A->rows);
     return launch<T>(KIND_FIXUP, mode, s, a, items, stream);
 }
 
@@ -641,9 +803,8 @@ using namespace cgnn;
 extern "C" size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dtype, int kernel) {
     if (A == nullptr || A->nnz <= 0 || F <= 0) return 0;
     if (resolve_kernel(A, kernel) == CGNN_SPMM_ROW) return 0;
-    const int64_t nseg = ceil_div(A->nnz, seg_len(A));
-    const size_t elt = dtype == CGNN_F64 ? 8 : 4;
-    return carry_row_bytes(nseg) + (size_t)nseg * (size_t)F * elt;
+    const int seg = seg_len(A);
+    return carry_levels(ceil_div(A->nnz, seg), F, dtype == CGNN_F64 ? 8 : 4, wants_levels(A, seg)).total;
 }
 
 extern "C" int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,

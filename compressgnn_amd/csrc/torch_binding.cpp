@@ -346,7 +346,7 @@ std::vector<Tensor> cluster_workspace(Tensor input, int64_t bits) {
 
 // Assignment and member lists of one refresh: ids [N] int64 (1-based), counts
 // [active+1] int32 (entry 0 = 0), active, and the member lists (offsets [active+2], perm
-// [N], sorted_id [N]).  The codes are grouped by a stable sort instead of bucket counters,
+// [N], sorted_id [N], and a host scalar with the size of the largest group).  The codes are grouped by a stable sort instead of bucket counters,
 // so the result is the same as cluster_assign_cuda's (cluster_kernel.cu:118-153) whatever
 // the distribution of the codes, and the member lists come with it.  The number of groups
 // is at most min(N, 2^bits): every kernel runs on buffers of that bound, so the device
@@ -366,12 +366,13 @@ std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(
     auto ints = input.options().dtype(torch::kInt32);
     Tensor ids = torch::empty({N}, input.options().dtype(torch::kInt64));
     Tensor perm = torch::empty({N}, ints), sorted_id = torch::empty({N}, ints);
+    auto host_scalar = [](int64_t v) { return torch::full({1}, v, torch::TensorOptions().dtype(torch::kInt64)); };
     if (N == 0)
-        return {ids, torch::zeros({1}, ints), 0, {torch::zeros({2}, ints), perm, sorted_id}};
+        return {ids, torch::zeros({1}, ints), 0, {torch::zeros({2}, ints), perm, sorted_id, host_scalar(0)}};
     const int64_t cap = std::min<int64_t>(N, n);
     Tensor raw = torch::empty({N}, ints);
     Tensor offsets = torch::empty({cap + 2}, ints), counts = torch::empty({cap + 1}, ints);
-    Tensor active_dev = torch::empty({1}, ints);
+    Tensor summary_dev = torch::empty({2}, ints);  // number of groups, largest group
     auto stream = current_stream(input);
     ok(cgnn_lsh_hash(N, input.size(1), (int)bits, dtype_code(input), input.data_ptr(), planes.data_ptr(),
                      raw.data_ptr<int32_t>(), nullptr, stream),
@@ -380,11 +381,12 @@ std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(
     Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, input.options().dtype(torch::kUInt8));
     ok(cgnn_lsh_group(N, (int)bits, raw.data_ptr<int32_t>(), ids.data_ptr<int64_t>(), offsets.data_ptr<int32_t>(),
                       perm.data_ptr<int32_t>(), sorted_id.data_ptr<int32_t>(), counts.data_ptr<int32_t>(),
-                      active_dev.data_ptr<int32_t>(), ws.data_ptr(), bytes, stream),
+                      summary_dev.data_ptr<int32_t>(), ws.data_ptr(), bytes, stream),
        "lsh_group");
-    const int active = active_dev.item<int>();
+    Tensor summary = summary_dev.cpu();  // the one host read of a refresh
+    const int active = summary.data_ptr<int32_t>()[0];
     return {ids, counts.narrow(0, 0, active + 1), (int64_t)active,
-            {offsets.narrow(0, 0, active + 2), perm, sorted_id}};
+            {offsets.narrow(0, 0, active + 2), perm, sorted_id, host_scalar(summary.data_ptr<int32_t>()[1])}};
 }
 
 // cluster_assign_cuda (cluster_kernel.cu:118-153).  The workspace of cluster_workspace is
@@ -450,7 +452,10 @@ std::vector<Tensor> members_or_build(const c10::optional<std::vector<Tensor>> &m
                                      int64_t groups) {
     if (members.has_value() && !members->empty()) {
         const auto &m = *members;
-        TORCH_CHECK(m.size() == 3 && m[0].numel() == groups + 1 && m[1].numel() == index.numel() &&
+        // an optional fourth entry: a host int64 scalar with the size of the largest group
+        TORCH_CHECK((m.size() == 3 || (m.size() == 4 && !m[3].is_cuda() && m[3].numel() == 1 &&
+                                       m[3].scalar_type() == torch::kInt64)) &&
+                        m[0].numel() == groups + 1 && m[1].numel() == index.numel() &&
                         m[2].numel() == index.numel() && m[0].scalar_type() == torch::kInt32 &&
                         m[1].scalar_type() == torch::kInt32 && m[2].scalar_type() == torch::kInt32 &&
                         m[0].device() == index.device(),
@@ -459,6 +464,8 @@ std::vector<Tensor> members_or_build(const c10::optional<std::vector<Tensor>> &m
     }
     return cluster_members(index, groups);
 }
+
+int64_t largest_group(const std::vector<Tensor> &m) { return m.size() == 4 ? m[3].item<int64_t>() : 0; }
 
 // cluster_mean_cuda (cluster_kernel.cu:158-170).  `members` (from cluster_members, for
 // the same index) avoids rebuilding the member lists on every call.
@@ -474,7 +481,7 @@ Tensor cluster_mean(Tensor input, Tensor index, Tensor count, c10::optional<std:
     Tensor out = torch::empty({groups, F}, input.options());
     const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(input));
     Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, input.options().dtype(torch::kUInt8));
-    ok(cgnn_cluster_mean(N, F, groups, dtype_code(input), input.data_ptr(), m[0].data_ptr<int32_t>(),
+    ok(cgnn_cluster_mean(N, F, groups, largest_group(m), dtype_code(input), input.data_ptr(), m[0].data_ptr<int32_t>(),
                          m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(), count.data_ptr<int32_t>(), out.data_ptr(),
                          ws.data_ptr(), bytes, current_stream(input)),
        "cluster_mean");
@@ -492,7 +499,7 @@ Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count, c10::optio
     if (out.numel() == 0) return out;
     const int32_t *perm = nullptr;
     if (members.has_value() && !members->empty()) {
-        TORCH_CHECK(members->size() == 3 && (*members)[1].numel() == index.numel() &&
+        TORCH_CHECK(members->size() >= 3 && (*members)[1].numel() == index.numel() &&
                         (*members)[1].scalar_type() == torch::kInt32 && (*members)[1].device() == index.device(),
                     "member lists do not match index");
         perm = (*members)[1].data_ptr<int32_t>();
@@ -518,7 +525,7 @@ Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias
     if (out.numel() == 0) return out;
     const int32_t *perm = nullptr;
     if (members.has_value() && !members->empty()) {
-        TORCH_CHECK(members->size() == 3 && (*members)[1].numel() == index.numel() &&
+        TORCH_CHECK(members->size() >= 3 && (*members)[1].numel() == index.numel() &&
                         (*members)[1].scalar_type() == torch::kInt32 && (*members)[1].device() == index.device(),
                     "member lists do not match index");
         perm = (*members)[1].data_ptr<int32_t>();
@@ -546,7 +553,7 @@ Tensor cluster_reconstruct_backward(Tensor grad, Tensor index, Tensor output, in
     Tensor out = torch::empty({groups, F}, grad.options());
     const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(grad));
     Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, grad.options().dtype(torch::kUInt8));
-    ok(cgnn_reconstruct_backward(N, F, groups, dtype_code(grad), grad.data_ptr(), output.data_ptr(),
+    ok(cgnn_reconstruct_backward(N, F, groups, largest_group(m), dtype_code(grad), grad.data_ptr(), output.data_ptr(),
                                  m[0].data_ptr<int32_t>(), m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(),
                                  relu ? 1 : 0, out.data_ptr(), ws.data_ptr(), bytes, current_stream(grad)),
        "cluster_reconstruct_backward");

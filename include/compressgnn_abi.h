@@ -148,19 +148,22 @@ int cgnn_cluster_members(int64_t N, int64_t groups, const int64_t *ids, int32_t 
  * counters): rows are sorted by code (stable), a run of equal codes is a group, and the
  * 1-based id of a group is the rank of its code.  Produces what cgnn_lsh_scan +
  * cgnn_lsh_finish + cgnn_cluster_members produce -- ids[N], counts[active+1] (entry 0 = 0),
- * offsets[active+2], perm[N], sorted_id[N] -- and *active (device scalar) = number of
- * groups.  counts needs room for min(N, 2^bits)+1 entries and offsets for one more; entries
+ * offsets[active+2], perm[N], sorted_id[N] -- and summary[2] (device): summary[0] = active,
+ * the number of groups, summary[1] = the size of the largest group.  counts needs room for min(N, 2^bits)+1 entries and offsets for one more; entries
  * beyond active+1 (active+2) are left untouched.  Replaces cluster_kernel.cu:143-150 and
  * the atomics of hash_ids (cluster_kernel.cu:41-59). */
 size_t cgnn_lsh_group_workspace_bytes(int64_t N, int bits);
 int cgnn_lsh_group(int64_t N, int bits, const int32_t *raw_code, int64_t *ids, int32_t *offsets,
-                   int32_t *perm, int32_t *sorted_id, int32_t *counts, int32_t *active,
+                   int32_t *perm, int32_t *sorted_id, int32_t *counts, int32_t *summary,
                    void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
 
 /* reps[g,:] = (sum over members i of group g, ascending i, of X[i,:]) / max(counts[g],1).
+ * max_members: size of the largest group if the caller knows it (it decides whether the
+ * sums of very large groups need the multi-level carry reduction), 0 if not.  The
+ * workspace size covers either case.
  * Replaces cluster_mean_cuda (cluster_kernel.cu:158-170). */
 size_t cgnn_cluster_mean_workspace_bytes(int64_t N, int64_t F, int64_t groups, int dtype);
-int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int dtype, const void *X,
+int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int64_t max_members, int dtype, const void *X,
                       const int32_t *offsets, const int32_t *perm, const int32_t *sorted_id,
                       const int32_t *counts, void *reps, void *workspace,
                       size_t workspace_bytes, cgnn_stream_t stream);
@@ -181,9 +184,9 @@ int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void
                      void *out, cgnn_stream_t stream);
 
 /* reps_grad[g,:] = sum over members i of g (ascending) of
- * ((relu && output[i,:] <= 0) ? 0 : grad[i,:]).
+ * ((relu && output[i,:] <= 0) ? 0 : grad[i,:]).  max_members as for cgnn_cluster_mean.
  * Replaces cluster_reconstruct_backward_cuda (cluster_kernel.cu:196-208). */
-int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int dtype, const void *grad,
+int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int64_t max_members, int dtype, const void *grad,
                               const void *output, const int32_t *offsets, const int32_t *perm,
                               const int32_t *sorted_id, int relu, void *reps_grad,
                               void *workspace, size_t workspace_bytes, cgnn_stream_t stream);

@@ -114,13 +114,15 @@ def test_grouped_assign_matches_counter_path(shape, bits):
     assert active == active0 == want_active
     assert np.array_equal(ids.cpu().numpy(), want_ids) and torch.equal(ids, ids0)
     assert np.array_equal(counts.cpu().numpy(), want_counts) and torch.equal(counts, counts0)
-    for got, ref in zip(members, members0):
+    for got, ref in zip(members[:3], members0):
         assert got.dtype == ref.dtype and torch.equal(got, ref)
+    assert members[3] == int(want_counts.max())
 
 
 def test_grouped_assign_empty():
     ids, counts, active, members = abi.lsh_assign_grouped(torch.zeros(0, 8, device=DEV), torch.randn(8, 8, device=DEV), 8)
     assert ids.numel() == 0 and active == 0 and counts.tolist() == [0] and members[0].tolist() == [0, 0]
+    assert members[3] == 0
 
 
 def test_assign_denormal_and_cancelling_projections():
@@ -191,6 +193,13 @@ def test_large_cluster_sums():
     np.testing.assert_allclose(reps, want64, rtol=1e-5, atol=1e-6)
     again = abi.cluster_mean(_t(x), members, counts).cpu().numpy()
     assert np.array_equal(reps, again)
+    # with the size of the largest group given, the chains of carries are known to be
+    # short enough for the serial fix-up alone; a wrong (too small) hint only costs time
+    largest = int(counts_np.max())
+    hinted = abi.cluster_mean(_t(x), members, counts, max_members=largest).cpu().numpy()
+    np.testing.assert_allclose(hinted, want64, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(abi.cluster_mean(_t(x), members, counts, max_members=1).cpu().numpy(), want64,
+                               rtol=1e-5, atol=1e-6)
     out = rng.standard_normal((n, F)).astype(np.float32)
     go = rng.standard_normal((n, F)).astype(np.float32)
     rg = abi.reconstruct_backward(_t(go), _t(out), members, 9, True).cpu().numpy()

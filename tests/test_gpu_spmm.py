@@ -71,6 +71,33 @@ def test_spmm_nnz_long_rows(F, seg):
     assert np.array_equal(got, again)
 
 
+@pytest.mark.parametrize("seg,F", [(8, 4), (8, 36), (64, 16), (64, 256)])
+def test_spmm_nnz_giant_rows(seg, F):
+    """Rows whose carries fill several levels of the carry reduction: one row with 300,000
+    entries next to rows of 1, 70, 5,000 and 40,000 entries, empty rows in between, and a
+    long row at the very end.  Checked against a float64 product (the giant rows are
+    summed in tree order, within the tolerance of the float32 path), fresh and
+    accumulating, and for run-to-run reproducibility."""
+    rng = np.random.default_rng(seg + F)
+    lens = [3, 300_000, 0, 1, 70, 0, 5_000, 40_000, 2, 0, 64, 65, 9_000]
+    cols = 5_000
+    vlist = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    elist = rng.integers(0, cols, size=int(vlist[-1])).astype(np.int64)
+    row_len = np.repeat(lens, lens)
+    value = (rng.standard_normal(len(elist)) * 0.3 / np.sqrt(row_len)).astype(np.float32)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    want = np.zeros((len(lens), F))
+    np.add.at(want, np.repeat(np.arange(len(lens)), lens), value[:, None].astype(np.float64) * x[elist])
+    got = _run(vlist, elist, value, x, abi.SPMM_NNZ, seg=seg)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=2e-5)
+    assert np.array_equal(got, _run(vlist, elist, value, x, abi.SPMM_NNZ, seg=seg))
+    assert not got[[2, 5, 9]].any()
+    out0 = rng.standard_normal((len(lens), F)).astype(np.float32)
+    got2 = _run(vlist, elist, value, x, abi.SPMM_NNZ, out0, seg=seg)
+    np.testing.assert_allclose(got2, want + out0, rtol=1e-4, atol=2e-5)
+    assert np.array_equal(got2[[2, 5, 9]], out0[[2, 5, 9]])
+
+
 @pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
 def test_spmm_edge_cases(kernel):
     rng = np.random.default_rng(5)
