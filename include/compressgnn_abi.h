@@ -197,6 +197,11 @@ int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int64_t max_
  * kernel for scaling profiler byte counters. */
 int cgnn_copy_bytes(const void *src, void *dst, size_t n, cgnn_stream_t stream);
 
+/* A plain streaming read of n bytes (n % 16 == 0) that stores nothing (sink: 4 bytes of
+ * device memory, practically never written): the read rate the memory system sustains,
+ * which is what the gather-bound kernels are compared with. */
+int cgnn_read_bytes(const void *src, size_t n, void *sink, cgnn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
