@@ -32,6 +32,7 @@ class CsrStruct(ctypes.Structure):
         ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("nnz", ctypes.c_int64),
         ("rowptr", ctypes.c_void_p), ("colidx", ctypes.c_void_p), ("rowidx", ctypes.c_void_p),
         ("val", ctypes.c_void_p), ("max_row_nnz", ctypes.c_int32), ("seg_nnz", ctypes.c_int32),
+        ("rowmap", ctypes.c_void_p),
     ]
 
 
@@ -86,16 +87,18 @@ def i64(x):
 class DeviceCsr:
     """A CSR block on the device with int32 indices (the layout the kernels read)."""
 
-    def __init__(self, rows, cols, rowptr, colidx, val, rowidx=None, max_row_nnz=0, seg_nnz=0):
+    def __init__(self, rows, cols, rowptr, colidx, val, rowidx=None, max_row_nnz=0, seg_nnz=0, rowmap=None):
         self.rows, self.cols = int(rows), int(cols)
         self.rowptr, self.colidx, self.val, self.rowidx = rowptr, colidx, val, rowidx
+        self.rowmap = rowmap  # int32 [rows] on the device: stored row g is row rowmap[g] of the output
         self.nnz = int(colidx.numel())
         self.max_row_nnz, self.seg_nnz = int(max_row_nnz), int(seg_nnz)
         self._ws = {}
 
     @classmethod
-    def from_host(cls, rows, cols, rowptr, colidx, val, device, with_rowidx=True, seg_nnz=0):
-        """rowptr/colidx: integer arrays or tensors on the host; val: float tensor/array or None."""
+    def from_host(cls, rows, cols, rowptr, colidx, val, device, with_rowidx=True, seg_nnz=0, rowmap=None):
+        """rowptr/colidx: integer arrays or tensors on the host; val: float tensor/array or None;
+        rowmap: the rows are given in a stored order, stored row g being output row rowmap[g]."""
         rp = torch.as_tensor(rowptr).to(torch.int64)
         ci = torch.as_tensor(colidx).to(torch.int64)
         lens = rp[1:] - rp[:-1]
@@ -104,8 +107,9 @@ class DeviceCsr:
         if with_rowidx:
             rowidx = torch.repeat_interleave(torch.arange(rows, dtype=torch.int32), lens).to(device)
         v = None if val is None else torch.as_tensor(val).to(device)
+        rm = None if rowmap is None else torch.as_tensor(rowmap).to(torch.int32).to(device)
         return cls(rows, cols, rp.to(torch.int32).to(device), ci.to(torch.int32).to(device), v, rowidx,
-                   max_row, seg_nnz)
+                   max_row, seg_nnz, rm)
 
     def struct(self):
         s = CsrStruct()
@@ -115,6 +119,7 @@ class DeviceCsr:
         s.rowidx = self.rowidx.data_ptr() if (self.rowidx is not None and self.nnz) else 0
         s.val = self.val.data_ptr() if (self.val is not None and self.nnz) else 0
         s.max_row_nnz, s.seg_nnz = self.max_row_nnz, self.seg_nnz
+        s.rowmap = self.rowmap.data_ptr() if self.rowmap is not None else 0
         return s
 
     def workspace(self, F, dtype, kernel):

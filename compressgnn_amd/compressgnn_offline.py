@@ -21,6 +21,7 @@ EXPORTS = [
     "cgnn_filter_csr", "cgnn_depth_filter_csr", "cgnn_gen_vertex_order_csr", "cgnn_gen_vertex_order_csc",
     "cgnn_compress_csr_batch", "cgnn_csr_hstack", "cgnn_csr_row_stats", "cgnn_gen_chung_lu", "cgnn_gen_copy_model",
     "cgnn_add_self_loop_coo", "cgnn_gcn_norm_coo_compress", "cgnn_gen_edge_order",
+    "cgnn_csr_locality_order", "cgnn_csr_permute_rows",
 ]
 
 _NP_TYPES = {0: np.int64, 1: np.float32, 2: np.int32}
@@ -261,6 +262,23 @@ def csr_hstack(a0, a1, col_offset):
     (v, e, w), _ = _take(lib().cgnn_csr_hstack(ctypes.c_int64(len(v0) - 1), _p(v0), _p(e0), _p(w0), _p(v1), _p(e1),
                                                _p(w1), ctypes.c_int64(col_offset)))
     return v, e, w
+
+
+def csr_locality_order(vlist, elist):
+    """Rows sorted lexicographically by their column lists (int32 [rows])."""
+    vlist, elist = _i64(vlist), _i64(elist)
+    (order,), _ = _take(lib().cgnn_csr_locality_order(ctypes.c_int64(len(vlist) - 1), _p(vlist), _p(elist)))
+    return order
+
+
+def csr_permute_rows(vlist, elist, value, order):
+    """(vlist, elist, value) with row g = row order[g] of the input; value may be None."""
+    vlist, elist = _i64(vlist), _i64(elist)
+    v = None if value is None else _f32(value)
+    order = np.ascontiguousarray(order, dtype=np.int32)
+    (nv, ne, nw), _ = _take(lib().cgnn_csr_permute_rows(ctypes.c_int64(len(vlist) - 1), _p(vlist), _p(elist), _p(v),
+                                                       _p(order)))
+    return nv, ne, (None if value is None else nw)
 
 
 def csr_row_stats(vlist):

@@ -9,11 +9,13 @@
 #include "compressgnn_prep.h"
 
 #include <algorithm>
+#include <climits>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <numeric>
+#include <parallel/algorithm>
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
@@ -895,6 +897,65 @@ cgnn_arrays *cgnn_compress_csr_batch(int64_t V, const int64_t *vlist, const int6
             return nullptr;
         }
     return guarded([&] { return compress_batch(V, vlist, elist, rounds, min_pair_frequency); });
+}
+
+cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const int64_t *elist) {
+    // Rows ordered lexicographically by their column lists (shorter list first on a common
+    // prefix, ties by row number): rows that gather the same columns end up next to each
+    // other, so that rows processed together find each other's gathers in cache.
+    if (rows < 0 || !vlist || rows >= (i64)INT32_MAX) {
+        set_error("csr_locality_order: bad arguments");
+        return nullptr;
+    }
+    return guarded([&] {
+        std::vector<int32_t> order((size_t)rows);
+        std::iota(order.begin(), order.end(), 0);
+        auto before = [&](int32_t a, int32_t b) {
+            const i64 *pa = elist + vlist[a], *ea = elist + vlist[a + 1];
+            const i64 *pb = elist + vlist[b], *eb = elist + vlist[b + 1];
+            for (; pa != ea && pb != eb; ++pa, ++pb)
+                if (*pa != *pb) return *pa < *pb;
+            if ((pa == ea) != (pb == eb)) return pa == ea;
+            return a < b;
+        };
+#ifdef _GLIBCXX_PARALLEL_PARALLEL_H
+        __gnu_parallel::sort(order.begin(), order.end(), before);
+#else
+        std::sort(order.begin(), order.end(), before);
+#endif
+        auto *out = new cgnn_arrays;
+        out->add(std::move(order));
+        return out;
+    });
+}
+
+cgnn_arrays *cgnn_csr_permute_rows(int64_t rows, const int64_t *vlist, const int64_t *elist, const float *value,
+                                   const int32_t *order) {
+    if (rows < 0 || !vlist || (rows > 0 && !order)) {
+        set_error("csr_permute_rows: bad arguments");
+        return nullptr;
+    }
+    return guarded([&] {
+        std::vector<i64> nv((size_t)rows + 1, 0), ne((size_t)vlist[rows]);
+        std::vector<float> nw(value ? (size_t)vlist[rows] : 0);
+        for (i64 g = 0; g < rows; ++g) {
+            const i64 r = order[g];
+            if (r < 0 || r >= rows) throw std::runtime_error("csr_permute_rows: order is not a permutation");
+            nv[g + 1] = nv[g] + (vlist[r + 1] - vlist[r]);
+        }
+        if (nv[rows] != vlist[rows]) throw std::runtime_error("csr_permute_rows: order is not a permutation");
+#pragma omp parallel for schedule(static)
+        for (i64 g = 0; g < rows; ++g) {
+            const i64 r = order[g];
+            std::copy(elist + vlist[r], elist + vlist[r + 1], ne.begin() + nv[g]);
+            if (value) std::copy(value + vlist[r], value + vlist[r + 1], nw.begin() + nv[g]);
+        }
+        auto *out = new cgnn_arrays;
+        out->add(std::move(nv));
+        out->add(std::move(ne));
+        out->add(std::move(nw));
+        return out;
+    });
 }
 
 cgnn_arrays *cgnn_csr_hstack(int64_t rows, const int64_t *vlist0, const int64_t *elist0, const float *value0,

@@ -39,6 +39,7 @@ namespace cgnn {
 namespace {
 
 constexpr int kUnroll = 8;        // gathers in flight per lane and tile
+constexpr int kXcds = 8;          // accelerator dies of an MI355X, each with its own L2
 constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
 
 enum { MODE_VAL = 0, MODE_UNIT = 1, MODE_RELU_MASK = 2, MODE_DUAL = 3 };
@@ -53,6 +54,7 @@ struct SpmmArgs {
     const int32_t *rowptr;
     const int32_t *colidx;
     const int32_t *rowidx;
+    const int32_t *rowmap;  // row schedule: stored row g is row rowmap[g] of Y (or NULL)
     const T *val;
     const T *X;   // gathered matrix (may alias Y)
     const T *X1;  // MODE_DUAL: source of the columns >= split
@@ -206,10 +208,19 @@ template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
     const int lane = threadIdx.x % LPR;
-    int row = blockIdx.x * GPB + threadIdx.x / LPR;
+    int block = blockIdx.x;
+    if (a.rowmap != nullptr) {
+        // Workgroups are dealt to the XCDs round robin; with a locality order the grid is a
+        // multiple of kXcds and XCD x takes the x-th contiguous share of the stored rows, so
+        // that neighbours in the order meet in one L2.
+        const int share = gridDim.x / kXcds;
+        block = (block % kXcds) * share + block / kXcds;
+    }
+    int row = block * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
     if (row >= a.rows) return;
     const int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
+    if (a.rowmap != nullptr) row = a.rowmap[row];  // from here on: the row of Y
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
     Acc<T, VEC, TILES, MODE> acc;
@@ -555,6 +566,7 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
     constexpr int GPB = kBlock / LPR;
     dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
     if (grid.x == 0) return CGNN_OK;
+    if (kind == KIND_ROW && a.rowmap != nullptr) grid.x = (unsigned)(ceil_div(grid.x, kXcds) * kXcds);
     switch (kind) {
         case KIND_ROW:
             if (mode == MODE_DUAL)
@@ -613,6 +625,7 @@ int launch(int kind, int mode, const Shape &s, const SpmmArgs<T> &a, int64_t ite
 }
 
 int resolve_kernel(const cgnn_csr *A, int kernel) {
+    if (A->rowmap != nullptr) return CGNN_SPMM_ROW;  // a locality order exists for the row schedule only
     if (kernel == CGNN_SPMM_ROW || kernel == CGNN_SPMM_NNZ) return kernel;
     // AUTO: rows are "near regular" when the longest one is a small multiple of the
     // mean; otherwise balance by non-zeros.  Needs rowidx for the nnz schedule.
@@ -650,6 +663,7 @@ SpmmArgs<T> make_args(const cgnn_csr *A, const void *X, const void *X1, int64_t 
     a.rowptr = A->rowptr;
     a.colidx = A->colidx;
     a.rowidx = A->rowidx;
+    a.rowmap = A->rowmap;
     a.val = static_cast<const T *>(A->val);
     a.X = static_cast<const T *>(X);
     a.X1 = static_cast<const T *>(X1);

@@ -47,6 +47,7 @@ void require_gpu(const Tensor &t, const char *name) {
 struct DeviceCsr {
     int64_t rows = 0, cols = 0, nnz = 0;
     Tensor rowptr, colidx, rowidx, val;
+    Tensor rowmap;  // optional: stored row g is output row rowmap[g]
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
     std::map<std::tuple<int64_t, int, int>, Tensor> scratch;
@@ -62,6 +63,7 @@ struct DeviceCsr {
         a.val = (nnz && val.defined()) ? val.data_ptr() : nullptr;
         a.max_row_nnz = max_row_nnz;
         a.seg_nnz = seg_nnz;
+        a.rowmap = rowmap.defined() ? rowmap.data_ptr<int32_t>() : nullptr;
         return a;
     }
 
@@ -82,7 +84,8 @@ struct DeviceCsr {
 
 // rowptr/col: int64 or int32 tensors on any device; value: float tensor or undefined.
 std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows,
-                                    int64_t cols, torch::Device device, int64_t seg_nnz) {
+                                    int64_t cols, torch::Device device, int64_t seg_nnz,
+                                    c10::optional<Tensor> rowmap = c10::nullopt) {
     TORCH_CHECK(device.is_cuda(), "DeviceCsr lives on a GPU");
     TORCH_CHECK(rowptr.dim() == 1 && col.dim() == 1 && rowptr.numel() == rows + 1, "rowptr must have rows+1 entries");
     auto blk = std::make_shared<DeviceCsr>();
@@ -118,6 +121,10 @@ std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Ten
     if (value.has_value() && value->defined()) {
         TORCH_CHECK(value->numel() == blk->nnz, "value must have one entry per non-zero");
         blk->val = value->to(device).contiguous();
+    }
+    if (rowmap.has_value() && rowmap->defined()) {
+        TORCH_CHECK(rowmap->dim() == 1 && rowmap->numel() == rows, "rowmap must have one entry per row");
+        blk->rowmap = rowmap->to(device).to(torch::kInt32).contiguous();
     }
     if (rows > 0) {
         Tensor lens = blk->rowptr.slice(0, 1, rows + 1) - blk->rowptr.slice(0, 0, rows);
@@ -586,11 +593,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("version", []() { return std::string(cgnn_version()); });
     py::class_<DeviceCsr, std::shared_ptr<DeviceCsr>>(m, "DeviceCsr")
         .def(py::init([](Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows, int64_t cols,
-                         torch::Device device, int64_t seg_nnz) {
-                 return make_csr(rowptr, col, value, rows, cols, device, seg_nnz);
+                         torch::Device device, int64_t seg_nnz, c10::optional<Tensor> rowmap) {
+                 return make_csr(rowptr, col, value, rows, cols, device, seg_nnz, rowmap);
              }),
              py::arg("rowptr"), py::arg("col"), py::arg("value"), py::arg("rows"), py::arg("cols"),
-             py::arg("device"), py::arg("seg_nnz") = 0)
+             py::arg("device"), py::arg("seg_nnz") = 0, py::arg("rowmap") = py::none())
+        .def_readonly("rowmap", &DeviceCsr::rowmap)
         .def_readonly("rows", &DeviceCsr::rows)
         .def_readonly("cols", &DeviceCsr::cols)
         .def_readonly("nnz", &DeviceCsr::nnz)

@@ -60,6 +60,12 @@ typedef struct cgnn_csr {
     const void *val;       /* [nnz] of the call's dtype, or NULL */
     int32_t max_row_nnz;   /* longest row, 0 if unknown (AUTO then picks NNZ) */
     int32_t seg_nnz;       /* NNZ schedule: non-zeros per lane group, 0 = default */
+    /* Optional row permutation (NULL = none).  The arrays above then describe the rows in
+     * a stored order chosen for locality (rows that gather the same columns next to each
+     * other): stored row g is row rowmap[g] of Y.  Results are unchanged.  Such a block
+     * always runs the ROW schedule, and its workgroups are numbered so that consecutive
+     * stored rows land on the same XCD (the eight L2 caches of an MI355X are private). */
+    const int32_t *rowmap; /* [rows] or NULL */
 } cgnn_csr;
 
 const char *cgnn_last_error(void);

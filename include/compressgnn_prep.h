@@ -117,6 +117,16 @@ cgnn_arrays *cgnn_csr_hstack(int64_t rows, const int64_t *vlist0, const int64_t 
                              const int64_t *vlist1, const int64_t *elist1, const float *value1,
                              int64_t col_offset);
 
+/* A row order for locality: rows sorted lexicographically by their column lists, so that
+ * rows which gather the same columns are neighbours.  -> [order (int32, rows)]: position g
+ * of the order holds row order[g]. */
+cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const int64_t *elist);
+
+/* The CSR with its rows rearranged: row g of the result is row order[g] of the input
+ * (value may be NULL).  -> [vlist, elist, value] */
+cgnn_arrays *cgnn_csr_permute_rows(int64_t rows, const int64_t *vlist, const int64_t *elist,
+                                   const float *value, const int32_t *order);
+
 /* Longest row, and a histogram of row lengths in powers of two:
  * hist[k] = rows with length in [2^(k-1), 2^k) for k >= 1, hist[0] = empty rows. */
 int cgnn_csr_row_stats(int64_t rows, const int64_t *vlist, int64_t *max_row, int64_t hist[40]);

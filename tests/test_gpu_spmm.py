@@ -189,6 +189,58 @@ def test_spmm_f64():
         np.testing.assert_allclose(Y.cpu().numpy(), want, rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("rows", [1, 7, 777, 4100])
+@pytest.mark.parametrize("F", [16, 128, 200])
+def test_spmm_stored_row_order(rows, F):
+    """A block whose rows are stored in another order (rowmap) gives the same bits as the
+    plain block, fresh, accumulating and in the two-source form; the locality order of the
+    host library is a permutation that sorts the rows by their column lists."""
+    from compressgnn_amd import compressgnn_offline as off
+    rng = np.random.default_rng(rows + F)
+    cols = 300
+    vlist, elist, value = random_csr(rng, rows, cols, 5.0)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    order = off.csr_locality_order(vlist, elist)
+    assert sorted(order.tolist()) == list(range(rows))
+    keys = [tuple(elist[vlist[r]:vlist[r + 1]]) for r in order]
+    assert keys == sorted(keys)
+    for perm in (order, rng.permutation(rows).astype(np.int32)):
+        pv, pe, pw = off.csr_permute_rows(vlist, elist, value, perm)
+        plain = abi.DeviceCsr.from_host(rows, cols, vlist, elist, value, DEV)
+        stored = abi.DeviceCsr.from_host(rows, cols, pv, pe, pw, DEV, rowmap=perm)
+        X = torch.from_numpy(x).to(DEV)
+        want = abi.spmm(plain, X, None, False, abi.SPMM_ROW)
+        got = abi.spmm(stored, X, None, False, abi.SPMM_AUTO)
+        assert torch.equal(got, want)
+        out0 = torch.from_numpy(rng.standard_normal((rows, F)).astype(np.float32)).to(DEV)
+        a, b = out0.clone(), out0.clone()
+        abi.spmm(plain, X, a, True, abi.SPMM_ROW)
+        abi.spmm(stored, X, b, True, abi.SPMM_NNZ)  # a stored order always runs the row schedule
+        assert torch.equal(a, b)
+        split = cols // 3
+        X0, X1 = X[:split].contiguous(), X[split:].contiguous()
+        assert torch.equal(abi.spmm_dual(stored, split, X0, X1, None, abi.SPMM_AUTO),
+                           abi.spmm_dual(plain, split, X0, X1, None, abi.SPMM_ROW))
+
+
+def test_spmm_f64_giant_row():
+    """Double precision through the carry reduction levels (a row of 120,000 entries at
+    8 entries per run)."""
+    rng = np.random.default_rng(23)
+    lens = [5, 120_000, 0, 33]
+    cols, F = 3_000, 6
+    vlist = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    elist = rng.integers(0, cols, size=int(vlist[-1])).astype(np.int64)
+    value = rng.standard_normal(len(elist)) / np.sqrt(np.repeat(lens, lens))
+    x = rng.standard_normal((cols, F))
+    want = np.zeros((len(lens), F))
+    np.add.at(want, np.repeat(np.arange(len(lens)), lens), value[:, None] * x[elist])
+    A = abi.DeviceCsr.from_host(len(lens), cols, vlist, elist, value, DEV, seg_nnz=8)
+    Y = abi.spmm(A, torch.from_numpy(x).to(DEV), None, False, abi.SPMM_NNZ)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(Y.cpu().numpy(), want, rtol=1e-11, atol=1e-12)
+
+
 def test_csr_prepare_i64():
     import ctypes
     rng = np.random.default_rng(19)
