@@ -203,24 +203,32 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
     return x;
 }
 
+// Row of Y that stored row r stands for.
+template <typename T>
+__device__ __forceinline__ int out_row(const SpmmArgs<T> &a, int r) {
+    return a.rowmap != nullptr ? a.rowmap[r] : r;
+}
+
+// Workgroups are dealt to the XCDs round robin.  With a locality order the grid is a multiple
+// of kXcds and XCD x takes the x-th contiguous share of the stored rows (or runs), so that
+// neighbours in the order meet in one L2.
+template <typename T>
+__device__ __forceinline__ int logical_block(const SpmmArgs<T> &a) {
+    if (a.rowmap == nullptr) return blockIdx.x;
+    const int share = gridDim.x / kXcds;
+    return (blockIdx.x % kXcds) * share + blockIdx.x / kXcds;
+}
+
 // ---------------------------------------------------------------- row schedule --
 template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
     const int lane = threadIdx.x % LPR;
-    int block = blockIdx.x;
-    if (a.rowmap != nullptr) {
-        // Workgroups are dealt to the XCDs round robin; with a locality order the grid is a
-        // multiple of kXcds and XCD x takes the x-th contiguous share of the stored rows, so
-        // that neighbours in the order meet in one L2.
-        const int share = gridDim.x / kXcds;
-        block = (block % kXcds) * share + block / kXcds;
-    }
-    int row = block * GPB + threadIdx.x / LPR;
+    int row = logical_block(a) * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
     if (row >= a.rows) return;
     const int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
-    if (a.rowmap != nullptr) row = a.rowmap[row];  // from here on: the row of Y
+    row = out_row(a, row);  // from here on: the row of Y
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
     Acc<T, VEC, TILES, MODE> acc;
@@ -267,7 +275,7 @@ template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
     const int lane = threadIdx.x % LPR;
-    int seg = blockIdx.x * GPB + threadIdx.x / LPR;
+    int seg = logical_block(a) * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
     if (seg >= a.nseg) return;
     const int e0 = run_boundary(a, seg * a.seg_nnz);
@@ -302,7 +310,7 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
             if (e + u < e1) {
                 if (r[u] != cur) {
                     // row `cur` ends inside this run: finish it here
-                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur, foff, acc, a.accumulate);
+                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
                     acc.clear();
                     cur = r[u];
                 }
@@ -322,7 +330,7 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
                 store_pack<T, VEC>(crow + foff[t], o);
             }
     } else {
-        write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur, foff, acc, a.accumulate);
+        write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
     }
     if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = continues ? cur : -1;
 }
@@ -384,7 +392,7 @@ __global__ __launch_bounds__(kBlock) void spmm_carry_reduce_kernel(SpmmArgs<T> a
                 // The one addition to these elements in this launch sequence (the row's
                 // last run has stored its part already), so its result does not depend on
                 // timing; sent as an atomic only so that the lane need not wait for Y.
-                T *y = a.Y + (int64_t)cur * a.F + f;
+                T *y = a.Y + (int64_t)out_row(a, cur) * a.F + f;
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) unsafeAtomicAdd(y + i, acc.v[i]);
                 return;
@@ -493,7 +501,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
                         for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
                 }
             }
-            T *y = a.Y + (int64_t)row * a.F + f;
+            T *y = a.Y + (int64_t)out_row(a, row) * a.F + f;
             Pack<T, VEC> o = load_pack<T, VEC>(y);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) o.v[i] = o.v[i] + acc.v[i];
@@ -506,7 +514,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
     for (int base = 0; base < n_empty; base += G) {
         const int src = deal_item<LPR>(empty, empty_rank, base, grp);
         if (src < 0) continue;
-        const int row = wave_item0 + src;
+        const int row = out_row(a, wave_item0 + src);
         Pack<T, VEC> zero;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) zero.v[i] = T(0);
@@ -566,7 +574,8 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
     constexpr int GPB = kBlock / LPR;
     dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
     if (grid.x == 0) return CGNN_OK;
-    if (kind == KIND_ROW && a.rowmap != nullptr) grid.x = (unsigned)(ceil_div(grid.x, kXcds) * kXcds);
+    if ((kind == KIND_ROW || kind == KIND_NNZ) && a.rowmap != nullptr)
+        grid.x = (unsigned)(ceil_div(grid.x, kXcds) * kXcds);
     switch (kind) {
         case KIND_ROW:
             if (mode == MODE_DUAL)
@@ -625,7 +634,6 @@ int launch(int kind, int mode, const Shape &s, const SpmmArgs<T> &a, int64_t ite
 }
 
 int resolve_kernel(const cgnn_csr *A, int kernel) {
-    if (A->rowmap != nullptr) return CGNN_SPMM_ROW;  // a locality order exists for the row schedule only
     if (kernel == CGNN_SPMM_ROW || kernel == CGNN_SPMM_NNZ) return kernel;
     // AUTO: rows are "near regular" when the longest one is a small multiple of the
     // mean; otherwise balance by non-zeros.  Needs rowidx for the nnz schedule.

@@ -62,9 +62,9 @@ typedef struct cgnn_csr {
     int32_t seg_nnz;       /* NNZ schedule: non-zeros per lane group, 0 = default */
     /* Optional row permutation (NULL = none).  The arrays above then describe the rows in
      * a stored order chosen for locality (rows that gather the same columns next to each
-     * other): stored row g is row rowmap[g] of Y.  Results are unchanged.  Such a block
-     * always runs the ROW schedule, and its workgroups are numbered so that consecutive
-     * stored rows land on the same XCD (the eight L2 caches of an MI355X are private). */
+     * other): stored row g is row rowmap[g] of Y.  Results are unchanged.  The workgroups
+     * of such a block are numbered so that consecutive stored rows land on the same XCD
+     * (the eight L2 caches of an MI355X are private). */
     const int32_t *rowmap; /* [rows] or NULL */
 } cgnn_csr;
 

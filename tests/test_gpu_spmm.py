@@ -215,7 +215,7 @@ def test_spmm_stored_row_order(rows, F):
         out0 = torch.from_numpy(rng.standard_normal((rows, F)).astype(np.float32)).to(DEV)
         a, b = out0.clone(), out0.clone()
         abi.spmm(plain, X, a, True, abi.SPMM_ROW)
-        abi.spmm(stored, X, b, True, abi.SPMM_NNZ)  # a stored order always runs the row schedule
+        abi.spmm(stored, X, b, True, abi.SPMM_NNZ)  # rows of at most one run: same bits in the nnz schedule
         assert torch.equal(a, b)
         split = cols // 3
         X0, X1 = X[:split].contiguous(), X[split:].contiguous()
