@@ -223,6 +223,33 @@ def test_spmm_stored_row_order(rows, F):
                            abi.spmm_dual(plain, split, X0, X1, None, abi.SPMM_ROW))
 
 
+@pytest.mark.parametrize("seg", [8, 64])
+def test_spmm_stored_row_order_long_rows(seg):
+    """Stored row order with rows that are cut into runs: carries, the carry reduction levels
+    and the fix-up pass all address the output through the row map."""
+    from compressgnn_amd import compressgnn_offline as off
+    rng = np.random.default_rng(seg)
+    lens = [4, 90_000, 0, 700, 1, 0, 33, 5_000, 66]
+    cols, F = 2_000, 20
+    vlist = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    elist = rng.integers(0, cols, size=int(vlist[-1])).astype(np.int64)
+    value = (rng.standard_normal(len(elist)) * 0.3 / np.sqrt(np.repeat(lens, lens))).astype(np.float32)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    want = np.zeros((len(lens), F))
+    np.add.at(want, np.repeat(np.arange(len(lens)), lens), value[:, None].astype(np.float64) * x[elist])
+    perm = rng.permutation(len(lens)).astype(np.int32)
+    pv, pe, pw = off.csr_permute_rows(vlist, elist, value, perm)
+    stored = abi.DeviceCsr.from_host(len(lens), cols, pv, pe, pw, DEV, seg_nnz=seg, rowmap=perm)
+    X = torch.from_numpy(x).to(DEV)
+    got = abi.spmm(stored, X, None, False, abi.SPMM_NNZ).cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=2e-5)
+    assert not got[[2, 5]].any()
+    out0 = rng.standard_normal((len(lens), F)).astype(np.float32)
+    Y = torch.from_numpy(out0.copy()).to(DEV)
+    abi.spmm(stored, X, Y, True, abi.SPMM_NNZ)
+    np.testing.assert_allclose(Y.cpu().numpy(), want + out0, rtol=1e-4, atol=2e-5)
+
+
 def test_spmm_f64_giant_row():
     """Double precision through the carry reduction levels (a row of 120,000 entries at
     8 entries per run)."""
