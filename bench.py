@@ -510,6 +510,20 @@ def main():
         log("[bench] CPU baseline (%s, %d threads): %.1f ms per step" % (kind, threads, ms_cpu))
 
     del plain, plain_t
+    # the same graph as per-phase edge lists (graph_type="coo"): forward + backward of the
+    # multi-phase form, beside the CompressGraph form timed above
+    from CompressgnnData import CompressgnnData
+    from CooPhases import CooPhasePlan
+    src = np.repeat(np.arange(C1_VERTICES, dtype=np.int64), np.diff(v_raw))
+    mask = np.zeros(1, dtype=bool)
+    coo = CompressgnnData(np.zeros((C1_VERTICES, 1), np.float32), (src, e_raw), np.zeros(1, np.int64), mask, mask, mask,
+                          add_self_loop=True, normalize=True, graph_type="coo").to(dev)
+    coo_plan = CooPhasePlan(coo.edge_index, coo.edge_weight, coo.vertex_cnt, coo.rule_cnt)
+    coo_ms = time_loop(lambda: (coo_plan.forward(x), coo_plan.backward(g)), args.steps, 2, torch)
+    detail["multi_phase_edge_lists_C1"] = dict(
+        phases=int(coo.step), ms_per_step=coo_ms,
+        max_abs_diff_vs_compress_graph=(coo_plan.forward(x) - out).abs().max().item())
+    del coo, coo_plan
     if not args.skip_cluster:
         torch.cuda.empty_cache()
         xc, planes = bench_cluster(torch, max(3, min(args.steps, 10)), detail)
