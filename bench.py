@@ -407,7 +407,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the hot path uses no "
-                 "collectives, see DESIGN.md for how it would shard)" % args.gpus)
+                 "collectives; it would shard by destination rows and by nodes)" % args.gpus)
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
