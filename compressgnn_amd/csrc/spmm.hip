@@ -15,10 +15,12 @@
 //   * nnz schedule  -- a lane group per run of about seg_nnz consecutive non-zeros (rows
 //     of any length cost the same).  Rows of at most seg_nnz entries always lie inside
 //     one run and are summed exactly as in the row schedule.  Longer rows are cut at
-//     multiples of seg_nnz: the part that continues into the next run is stored as a
-//     carry row.  The carries of one row are consecutive; spmm_carry_reduce_kernel sums
-//     them 64 at a time, level by level (a row with a million entries is not walked by
-//     one lane group), and spmm_fixup_kernel adds what is left, in ascending order.
+//     multiples of seg_nnz: the part that continues into the next run is a carry.  The
+//     lane groups of one workgroup first add their carries of the same row in LDS, in
+//     ascending order, so at most one carry row per output row and workgroup reaches
+//     memory.  spmm_carry_reduce_kernel sums the carries of very long rows 64 at a
+//     time, level by level (a row with a million entries is not walked by one lane
+//     group), and spmm_fixup_kernel adds what is left, in ascending order.
 //     Every output element receives its additions in a fixed order (where an atomic add
 //     is used it is the only addition to that element), so results are reproducible run
 //     to run.
@@ -71,7 +73,15 @@ struct SpmmArgs {
     int32_t seg_nnz;
     int32_t split;
     int32_t accumulate;
+    // Runs per workgroup of the nnz kernel that wrote carry_row/carry (its carries are
+    // merged per workgroup: see kMerged), or 1 for the plain list a reduction level writes.
+    int32_t merge_stride;
 };
+
+// carry_row values below zero: the run carries nothing, or its carry was added to that
+// of an earlier run of the same workgroup (the row of Y is the one of that earlier run).
+constexpr int kNoCarry = -1;
+constexpr int kMerged = -2;
 
 template <typename T, int VEC>
 __device__ __forceinline__ Pack<T, VEC> load_pack(const T *p) {
@@ -274,69 +284,97 @@ __device__ __forceinline__ int run_boundary(const SpmmArgs<T> &a, int e) {
 template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
-    const int lane = threadIdx.x % LPR;
-    int seg = logical_block(a) * GPB + threadIdx.x / LPR;
+    __shared__ int wg_row[GPB];
+    __shared__ Pack<T, VEC> wg_carry[TILES][kBlock];
+    const int lane = threadIdx.x % LPR, grp = threadIdx.x / LPR;
+    int seg = logical_block(a) * GPB + grp;
     if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
-    if (seg >= a.nseg) return;
-    const int e0 = run_boundary(a, seg * a.seg_nnz);
-    const int e1 = run_boundary(a, (seg + 1) * a.seg_nnz);
-    if (e0 >= e1) {  // cannot happen for a well-formed CSR; keeps the fix-up pass consistent
-        if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = -1;
-        return;
+    int e0 = 0, e1 = 0;
+    if (seg < a.nseg) {
+        e0 = run_boundary(a, seg * a.seg_nnz);
+        e1 = run_boundary(a, (seg + 1) * a.seg_nnz);
     }
+    // e0 >= e1 inside the list cannot happen for a well-formed CSR
+    const bool active = e0 < e1;
     int64_t foff[TILES];
     feature_offsets<VEC, LPR, TILES>(a.F, lane, foff);
     Acc<T, VEC, TILES, MODE> acc;
     acc.clear();
-    int cur = a.rowidx[e0];
-    for (int e = e0; e < e1; e += kUnroll) {
-        int r[kUnroll], c[kUnroll];
-        T w[kUnroll];
-        Pack<T, VEC> x[kUnroll][TILES];
+    int cur = -1;
+    bool continues = false;
+    if (active) {
+        cur = a.rowidx[e0];
+        for (int e = e0; e < e1; e += kUnroll) {
+            int r[kUnroll], c[kUnroll];
+            T w[kUnroll];
+            Pack<T, VEC> x[kUnroll][TILES];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int idx = min(e + u, e1 - 1);
-            r[u] = a.rowidx[idx];
-            c[u] = a.colidx[idx];
-            if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
-            else w[u] = T(1);
-        }
+            for (int u = 0; u < kUnroll; ++u) {
+                const int idx = min(e + u, e1 - 1);
+                r[u] = a.rowidx[idx];
+                c[u] = a.colidx[idx];
+                if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
+                else w[u] = T(1);
+            }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
-            for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
+                for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            if (e + u < e1) {
-                if (r[u] != cur) {
-                    // row `cur` ends inside this run: finish it here
-                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
-                    acc.clear();
-                    cur = r[u];
+            for (int u = 0; u < kUnroll; ++u) {
+                if (e + u < e1) {
+                    if (r[u] != cur) {
+                        // row `cur` ends inside this run: finish it here
+                        write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+                        acc.clear();
+                        cur = r[u];
+                    }
+                    acc.add(x[u], w[u], c[u] >= a.split);
                 }
-                acc.add(x[u], w[u], c[u] >= a.split);
             }
         }
+        continues = (e1 < a.nnz) && (a.rowidx[e1] == cur);
+        if (!continues) write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
     }
-    const bool continues = (e1 < a.nnz) && (a.rowidx[e1] == cur);
+    // The carries of one row are added per workgroup: the first of its lane groups that
+    // carries the row takes those of the groups behind it, in ascending order.
+    Pack<T, VEC> part[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[t].v[i] = acc.total(T(0), t, i);
+    if (lane == 0) wg_row[grp] = continues ? cur : kNoCarry;
     if (continues) {
-        T *crow = a.carry + (int64_t)seg * a.F;
 #pragma unroll
-        for (int t = 0; t < TILES; ++t)
-            if (foff[t] >= 0) {
-                Pack<T, VEC> o;
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) o.v[i] = acc.total(T(0), t, i);
-                store_pack<T, VEC>(crow + foff[t], o);
-            }
-    } else {
-        write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+        for (int t = 0; t < TILES; ++t) wg_carry[t][threadIdx.x] = part[t];
     }
-    if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = continues ? cur : -1;
+    __syncthreads();
+    if (seg >= a.nseg) return;
+    int mark = kNoCarry;
+    if (continues) {
+        const bool first = grp == 0 || wg_row[grp - 1] != cur;
+        mark = first ? cur : kMerged;
+        if (first) {
+            for (int g = grp + 1; g < GPB && wg_row[g] == cur; ++g)
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) {
+                    const Pack<T, VEC> o = wg_carry[t][g * LPR + lane];
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) part[t].v[i] = part[t].v[i] + o.v[i];
+                }
+            T *crow = a.carry + (int64_t)seg * a.F;
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+                if (foff[t] >= 0) store_pack<T, VEC>(crow + foff[t], part[t]);
+        }
+    }
+    if (lane == 0 && blockIdx.y == 0) a.carry_row[seg] = mark;
 }
 
-// One level of the carry reduction.  Carries (row, vector) with equal rows are adjacent;
-// -1 marks a run that carries nothing.  A lane group takes kCarryFan consecutive carries:
+// One level of the carry reduction.  Carries (row, vector) with equal rows are adjacent
+// (in the list the nnz kernel writes, kMerged entries may lie between them: they are
+// skipped); kNoCarry marks a run that carries nothing.  A lane group takes kCarryFan
+// consecutive carries:
 // a row whose carries all lie inside the chunk is finished here (Y += their sum, nobody
 // else touches that row); the part of a row that reaches the chunk from before goes to
 // slot 2*chunk of the next level, the part of a row that goes on behind the chunk to slot
@@ -354,7 +392,8 @@ __global__ __launch_bounds__(kBlock) void spmm_carry_reduce_kernel(SpmmArgs<T> a
     const int s0 = chunk * kCarryFan;
     if (s0 >= a.nseg) return;
     const int s1 = min(s0 + kCarryFan, a.nseg);
-    const int before = s0 > 0 ? a.carry_row[s0 - 1] : -1;
+    const bool merged = a.merge_stride > 1;  // the list of the nnz kernel: s0 starts a workgroup
+    const int before = (s0 > 0 && !merged) ? a.carry_row[s0 - 1] : -1;
     const int after = s1 < a.nseg ? a.carry_row[s1] : -1;
     // the rows of the chunk: every lane of the group reads all of them (same addresses,
     // one round trip), so no lane has to wait for another
@@ -417,11 +456,14 @@ __global__ __launch_bounds__(kBlock) void spmm_carry_reduce_kernel(SpmmArgs<T> a
                 c[u] = rr[b + u] >= 0 ? load_pack<T, VEC>(a.carry + (int64_t)(s0 + b + u) * a.F + f) : zero;
 #pragma unroll
             for (int u = 0; u < kReduceBatch; ++u) {
-                if (rr[b + u] != cur) {  // entries behind the end of the last chunk are -1
+                if (rr[b + u] != cur && rr[b + u] != kMerged) {  // entries behind the end of the last chunk are -1
                     close(true);
                     cur = rr[b + u];
                     acc = zero;
-                    from_before = (b + u == 0) && cur >= 0 && cur == before;
+                    // is the row carried into the chunk?  In the list of the nnz kernel the
+                    // run before s0 may be a merged one, so ask where the row starts.
+                    from_before = (b + u == 0) && cur >= 0 &&
+                                  (merged ? (int64_t)a.rowptr[cur] < (int64_t)s0 * a.seg_nnz : cur == before);
                 }
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
@@ -436,11 +478,11 @@ __global__ __launch_bounds__(kBlock) void spmm_carry_reduce_kernel(SpmmArgs<T> a
 }
 
 // Adds the carries of every row that straddles runs, in ascending run order, and
-// (when not accumulating) clears the rows that have no entries.  One thread looks at
-// one work item: item i < nseg is run i, which matters if it holds the first carry of
-// its row; item i < rows is row i, which matters if it is empty (the two sets of rows
-// are disjoint).  The items of a wave that matter are then dealt out to its lane groups
-// (LPR lanes across the features), kFixBatch carry rows in flight per group.
+// (when not accumulating) clears the rows that have no entries (the two sets of rows are
+// disjoint).  Carries: one lane group (LPR lanes across the features) per run; the group
+// whose run holds the first carry of a row walks the row's carries, kFixBatch in flight,
+// and adds their sum to the row.  Empty rows: one thread looks at one row, and the empty
+// rows of a wave are then dealt out to its lane groups.
 
 // Lane (within the wave) of the flagged item this lane's group should handle in the
 // round that starts at rank `base`, or -1.  Uniform control flow: every lane calls it.
@@ -458,44 +500,49 @@ __device__ __forceinline__ int deal_item(bool flag, int my_rank, int base, int g
 
 template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
-    constexpr int G = kWave / LPR;
+    constexpr int GPB = kBlock / LPR;
     const int lane = threadIdx.x % kWave;
     const int sub = lane % LPR, grp = lane / LPR;
-    const int item = blockIdx.x * kBlock + threadIdx.x;
-    const int wave_item0 = item - lane;
-    int r = -1;
-    bool head = false;
-    if (item < a.nseg) {
-        r = a.carry_row[item];
-        head = r >= 0 && (item == 0 || a.carry_row[item - 1] != r);
-    }
-    const bool empty = !a.accumulate && item < a.rows && a.rowptr[item] == a.rowptr[item + 1];
-    const unsigned long long below = (1ull << lane) - 1ull;
 
-    const unsigned long long heads = __ballot(head);
-    const int n_heads = __popcll(heads), head_rank = __popcll(heads & below);
-    for (int base = 0; base < n_heads; base += G) {
-        const int src = deal_item<LPR>(head, head_rank, base, grp);
-        const int row = __shfl(r, src < 0 ? 0 : src, kWave);
-        if (src < 0) continue;
-        const int s0 = wave_item0 + src;
+    int s0 = blockIdx.x * GPB + threadIdx.x / LPR;
+    if constexpr (LPR == kWave) s0 = __builtin_amdgcn_readfirstlane(s0);
+    const int stride = a.merge_stride > 1 ? a.merge_stride : 1;
+    int row = -1;
+    if (s0 < a.nseg) {
+        const int r = a.carry_row[s0];
+        // first carry of its row?  The list of the nnz kernel holds one carry per row and
+        // workgroup (every `stride` runs), and a row has an earlier carry exactly when it
+        // starts before this run; in a plain list the carries of a row are adjacent.
+        if (r >= 0) {
+            const bool head = stride > 1 ? (int64_t)a.rowptr[r] >= (int64_t)s0 * a.seg_nnz
+                                         : (s0 == 0 || a.carry_row[s0 - 1] != r);
+            if (head) row = r;
+        }
+    }
+    if (row >= 0) {
+        // the row's carries: the one at s0, then one per `stride` entries from the next
+        // multiple of `stride` on
+        const int64_t group0 = (int64_t)(s0 / stride) * stride;
         for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC) {
             Pack<T, VEC> acc;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc.v[i] = T(0);
             bool more = true;
-            for (int s = s0; more; s += kFixBatch) {
+            for (int k = 0; more; k += kFixBatch) {
                 int rr[kFixBatch];
+                bool inside[kFixBatch];
                 Pack<T, VEC> c[kFixBatch];
 #pragma unroll
                 for (int u = 0; u < kFixBatch; ++u) {
-                    const int idx = min(s + u, a.nseg - 1);
+                    const int64_t p = (k + u == 0) ? (int64_t)s0 : group0 + (int64_t)(k + u) * stride;
+                    inside[u] = p < a.nseg;
+                    const int64_t idx = inside[u] ? p : (int64_t)a.nseg - 1;
                     rr[u] = a.carry_row[idx];
-                    c[u] = load_pack<T, VEC>(a.carry + (int64_t)idx * a.F + f);
+                    c[u] = load_pack<T, VEC>(a.carry + idx * a.F + f);
                 }
 #pragma unroll
                 for (int u = 0; u < kFixBatch; ++u) {
-                    more = more && (s + u < a.nseg) && (rr[u] == row);
+                    more = more && inside[u] && (rr[u] == row);
                     if (more)
 #pragma unroll
                         for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
@@ -509,17 +556,24 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
         }
     }
 
+    if (a.accumulate) return;
+    const int item = blockIdx.x * kBlock + threadIdx.x;
+    const int wave_item0 = item - lane;
+    if (wave_item0 >= a.rows) return;
+    const bool empty = item < a.rows && a.rowptr[item] == a.rowptr[item + 1];
+    const unsigned long long below = (1ull << lane) - 1ull;
     const unsigned long long empties = __ballot(empty);
     const int n_empty = __popcll(empties), empty_rank = __popcll(empties & below);
+    constexpr int G = kWave / LPR;
     for (int base = 0; base < n_empty; base += G) {
         const int src = deal_item<LPR>(empty, empty_rank, base, grp);
         if (src < 0) continue;
-        const int row = out_row(a, wave_item0 + src);
+        const int erow = out_row(a, wave_item0 + src);
         Pack<T, VEC> zero;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) zero.v[i] = T(0);
         for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC)
-            store_pack_stream<T, VEC>(a.Y + (int64_t)row * a.F + f, zero);
+            store_pack_stream<T, VEC>(a.Y + (int64_t)erow * a.F + f, zero);
     }
 }
 
@@ -593,9 +647,14 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
             else
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_RELU_MASK>), grid, block, 0, stream, a);
             break;
-        case KIND_FIXUP:
-            hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, kBlock)), block, 0, stream, a);
+        case KIND_FIXUP: {  // a lane group per carry, and (when not accumulating) a thread per row
+            const int64_t for_rows = a.accumulate ? 0 : ceil_div((int64_t)a.rows, kBlock);
+            const int64_t for_carries = ceil_div((int64_t)a.nseg, GPB);
+            const int64_t n = for_rows > for_carries ? for_rows : for_carries;
+            if (n > 0)
+                hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR>), dim3((unsigned)n), block, 0, stream, a);
             break;
+        }
         case KIND_REDUCE:  // items = chunks of kCarryFan carries, one lane group each
             hipLaunchKernelGGL((spmm_carry_reduce_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, GPB)), block, 0,
                                stream, a);
@@ -753,6 +812,8 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     a.carry_row = nseg > 0 ? level_rows(0) : nullptr;
     a.carry = nseg > 0 ? level_carries(0) : nullptr;
     Shape s = pick_shape<T>(F, X, Y, a.carry, mode == MODE_DUAL ? X1 : M);
+    const int runs_per_workgroup = kBlock / s.lpr;
+    a.merge_stride = runs_per_workgroup;
     if (nseg > 0) {
         int rc = launch<T>(KIND_NNZ, mode, s, a, nseg, stream);
         if (rc != CGNN_OK) return rc;
@@ -763,6 +824,7 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
         a.carry = level_carries(k);
         a.carry_row_out = level_rows(k + 1);
         a.carry_out = level_carries(k + 1);
+        a.merge_stride = k == 0 ? runs_per_workgroup : 1;
         int rc = launch<T>(KIND_REDUCE, mode, s, a, ceil_div(levels.n[k], kCarryFan), stream);
         if (rc != CGNN_OK) return rc;
     }
@@ -771,6 +833,7 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
         a.nseg = (int32_t)levels.n[last];
         a.carry_row = level_rows(last);
         a.carry = level_carries(last);
+        a.merge_stride = last == 0 ? runs_per_workgroup : 1;
     }
     const int64_t items = accumulate ? a.nseg : (a.nseg > A->rows ? a.nseg : A->rows);
     return launch<T>(KIND_FIXUP, mode, s, a, items, stream);
