@@ -498,51 +498,71 @@ __device__ __forceinline__ int deal_item(bool flag, int my_rank, int base, int g
     return src;
 }
 
-template <typename T, int VEC, int LPR>
+template <typename T, int VEC, int LPR, bool MERGED>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
+    // carry rows in flight per lane group; few, so that the many groups that find nothing
+    // to do are all resident at once
+    constexpr int BATCH = MERGED ? 4 : kFixBatch;
     const int lane = threadIdx.x % kWave;
     const int sub = lane % LPR, grp = lane / LPR;
 
     int s0 = blockIdx.x * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) s0 = __builtin_amdgcn_readfirstlane(s0);
-    const int stride = a.merge_stride > 1 ? a.merge_stride : 1;
-    int row = -1;
+    const int stride = MERGED ? a.merge_stride : 1;  // MERGED: the list of the nnz kernel
+    // First carry of its row?  The list of the nnz kernel holds one carry per row and
+    // workgroup: a row has an earlier carry exactly when it starts before this run, and
+    // its later carries belong to the first run of every following workgroup whose end
+    // still lies inside the row.  In a plain list the carries of a row are adjacent.
+    int row = -1, row_end = 0;
     if (s0 < a.nseg) {
         const int r = a.carry_row[s0];
-        // first carry of its row?  The list of the nnz kernel holds one carry per row and
-        // workgroup (every `stride` runs), and a row has an earlier carry exactly when it
-        // starts before this run; in a plain list the carries of a row are adjacent.
         if (r >= 0) {
-            const bool head = stride > 1 ? (int64_t)a.rowptr[r] >= (int64_t)s0 * a.seg_nnz
-                                         : (s0 == 0 || a.carry_row[s0 - 1] != r);
+            bool head;
+            if constexpr (MERGED) {
+                head = (int64_t)a.rowptr[r] >= (int64_t)s0 * a.seg_nnz;
+                row_end = a.rowptr[r + 1];
+            } else {
+                head = s0 == 0 || a.carry_row[s0 - 1] != r;
+            }
             if (head) row = r;
         }
     }
     if (row >= 0) {
-        // the row's carries: the one at s0, then one per `stride` entries from the next
-        // multiple of `stride` on
         const int64_t group0 = (int64_t)(s0 / stride) * stride;
+#pragma unroll 1
         for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC) {
-            Pack<T, VEC> acc;
+            Pack<T, VEC> acc, zero;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) acc.v[i] = T(0);
+            for (int i = 0; i < VEC; ++i) acc.v[i] = zero.v[i] = T(0);
             bool more = true;
-            for (int k = 0; more; k += kFixBatch) {
-                int rr[kFixBatch];
-                bool inside[kFixBatch];
-                Pack<T, VEC> c[kFixBatch];
+#pragma unroll 1
+            for (int k = 0; more; k += BATCH) {
+                bool take[BATCH];
+                Pack<T, VEC> c[BATCH];
+                if constexpr (MERGED) {
 #pragma unroll
-                for (int u = 0; u < kFixBatch; ++u) {
-                    const int64_t p = (k + u == 0) ? (int64_t)s0 : group0 + (int64_t)(k + u) * stride;
-                    inside[u] = p < a.nseg;
-                    const int64_t idx = inside[u] ? p : (int64_t)a.nseg - 1;
-                    rr[u] = a.carry_row[idx];
-                    c[u] = load_pack<T, VEC>(a.carry + idx * a.F + f);
+                    for (int u = 0; u < BATCH; ++u) {
+                        const int64_t p = (k + u == 0) ? (int64_t)s0 : group0 + (int64_t)(k + u) * stride;
+                        take[u] = (k + u == 0) || (p + 1) * a.seg_nnz < (int64_t)row_end;
+                        c[u] = take[u] ? load_pack<T, VEC>(a.carry + p * a.F + f) : zero;
+                    }
+                } else {
+                    int rr[BATCH];
+#pragma unroll
+                    for (int u = 0; u < BATCH; ++u) {
+                        const int64_t p = (int64_t)s0 + k + u;
+                        take[u] = p < a.nseg;
+                        const int64_t idx = take[u] ? p : (int64_t)a.nseg - 1;
+                        rr[u] = a.carry_row[idx];
+                        c[u] = load_pack<T, VEC>(a.carry + idx * a.F + f);
+                    }
+#pragma unroll
+                    for (int u = 0; u < BATCH; ++u) take[u] = take[u] && rr[u] == row;
                 }
 #pragma unroll
-                for (int u = 0; u < kFixBatch; ++u) {
-                    more = more && inside[u] && (rr[u] == row);
+                for (int u = 0; u < BATCH; ++u) {
+                    more = more && take[u];
                     if (more)
 #pragma unroll
                         for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
@@ -650,9 +670,11 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
         case KIND_FIXUP: {  // a lane group per carry, and (when not accumulating) a thread per row
             const int64_t for_rows = a.accumulate ? 0 : ceil_div((int64_t)a.rows, kBlock);
             const int64_t for_carries = ceil_div((int64_t)a.nseg, GPB);
-            const int64_t n = for_rows > for_carries ? for_rows : for_carries;
-            if (n > 0)
-                hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR>), dim3((unsigned)n), block, 0, stream, a);
+            const dim3 fix_grid((unsigned)(for_rows > for_carries ? for_rows : for_carries));
+            if (fix_grid.x > 0 && a.merge_stride > 1)
+                hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR, true>), fix_grid, block, 0, stream, a);
+            else if (fix_grid.x > 0)  // the short list a reduction level leaves
+                hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR, false>), fix_grid, block, 0, stream, a);
             break;
         }
         case KIND_REDUCE:  // items = chunks of kCarryFan carries, one lane group each
@@ -757,12 +779,12 @@ struct CarryLevels {
     size_t total = 0;
 };
 
-// Rows known to span fewer than kLongChain runs need no reduction levels: the fix-up
-// pass walks such chains directly.  max_row_nnz == 0 means unknown.
-constexpr int64_t kLongChain = 1024;
+// Rows whose carries the fix-up pass can walk directly (at most kLongChain of them, one per
+// workgroup of the nnz kernel) need no reduction levels.  max_row_nnz == 0 means unknown.
+constexpr int64_t kLongChain = 256;
 
-bool wants_levels(const cgnn_csr *A, int seg) {
-    return A->max_row_nnz <= 0 || (int64_t)A->max_row_nnz > kLongChain * seg;
+bool wants_levels(const cgnn_csr *A, int seg, int runs_per_workgroup) {
+    return A->max_row_nnz <= 0 || (int64_t)A->max_row_nnz > kLongChain * seg * runs_per_workgroup;
 }
 
 CarryLevels carry_levels(int64_t nseg, int64_t F, size_t elt, bool reduce) {
@@ -799,7 +821,11 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     if (A->nnz > 0 && A->rowidx == nullptr) return fail(CGNN_EINVAL, "spmm: nnz schedule needs rowidx");
     const int seg = seg_len(A);
     const int64_t nseg = ceil_div(A->nnz, seg);
-    const CarryLevels levels = carry_levels(nseg, F, sizeof(T), wants_levels(A, seg));
+    // the lane layout decides how many runs a workgroup merges (the carries sit at multiples
+    // of 256 bytes in the workspace, so the workspace stands for them in the alignment check)
+    const Shape s = pick_shape<T>(F, X, Y, ws, mode == MODE_DUAL ? X1 : M);
+    const int runs_per_workgroup = kBlock / s.lpr;
+    const CarryLevels levels = carry_levels(nseg, F, sizeof(T), wants_levels(A, seg, runs_per_workgroup));
     if (nseg > 0 && (ws == nullptr || ws_bytes < levels.total)) {
         set_error("spmm: workspace of %zu bytes needed, %zu given", levels.total, ws_bytes);
         return CGNN_EWORKSPACE;
@@ -811,8 +837,6 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     a.seg_nnz = seg;
     a.carry_row = nseg > 0 ? level_rows(0) : nullptr;
     a.carry = nseg > 0 ? level_carries(0) : nullptr;
-    Shape s = pick_shape<T>(F, X, Y, a.carry, mode == MODE_DUAL ? X1 : M);
-    const int runs_per_workgroup = kBlock / s.lpr;
     a.merge_stride = runs_per_workgroup;
     if (nseg > 0) {
         int rc = launch<T>(KIND_NNZ, mode, s, a, nseg, stream);
@@ -889,7 +913,9 @@ extern "C" size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dt
     if (A == nullptr || A->nnz <= 0 || F <= 0) return 0;
     if (resolve_kernel(A, kernel) == CGNN_SPMM_ROW) return 0;
     const int seg = seg_len(A);
-    return carry_levels(ceil_div(A->nnz, seg), F, dtype == CGNN_F64 ? 8 : 4, wants_levels(A, seg)).total;
+    // an upper bound: the lane layout (which depends on the pointers' alignment) can only
+    // remove reduction levels
+    return carry_levels(ceil_div(A->nnz, seg), F, dtype == CGNN_F64 ? 8 : 4, wants_levels(A, seg, 1)).total;
 }
 
 extern "C" int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
