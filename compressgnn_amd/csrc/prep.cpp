@@ -899,17 +899,25 @@ cgnn_arrays *cgnn_compress_csr_batch(int64_t V, const int64_t *vlist, const int6
     return guarded([&] { return compress_batch(V, vlist, elist, rounds, min_pair_frequency); });
 }
 
+// Columns listed by more rows than this are left out when rows are matched by the columns
+// they share: nearly every pair of rows shares such a column (and it stays in cache anyway).
+static const i64 kLocalityHubRows = 256;
+
 cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const int64_t *elist) {
-    // Rows ordered lexicographically by their column lists (shorter list first on a common
-    // prefix, ties by row number): rows that gather the same columns end up next to each
-    // other, so that rows processed together find each other's gathers in cache.
+    // Rows that gather the same columns should be processed one after the other, so that
+    // they find each other's gathers in cache.  Every row is tied to the row it shares most
+    // columns with (ties: the lower row); the ties that close no cycle form a forest, and
+    // the order is a depth-first walk of it, closest relatives first.  Trees are entered
+    // in the lexicographic order of the column lists (shorter list first on a common
+    // prefix, then by row number), which also orders the rows that share nothing.
     if (rows < 0 || !vlist || rows >= (i64)INT32_MAX) {
         set_error("csr_locality_order: bad arguments");
         return nullptr;
     }
     return guarded([&] {
-        std::vector<int32_t> order((size_t)rows);
-        std::iota(order.begin(), order.end(), 0);
+        const i64 nnz = vlist[rows];
+        std::vector<int32_t> lex((size_t)rows);
+        std::iota(lex.begin(), lex.end(), 0);
         auto before = [&](int32_t a, int32_t b) {
             const i64 *pa = elist + vlist[a], *ea = elist + vlist[a + 1];
             const i64 *pb = elist + vlist[b], *eb = elist + vlist[b + 1];
@@ -919,10 +927,113 @@ cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const i
             return a < b;
         };
 #ifdef _GLIBCXX_PARALLEL_PARALLEL_H
-        __gnu_parallel::sort(order.begin(), order.end(), before);
+        __gnu_parallel::sort(lex.begin(), lex.end(), before);
 #else
-        std::sort(order.begin(), order.end(), before);
+        std::sort(lex.begin(), lex.end(), before);
 #endif
+        // column -> rows that list it
+        i64 cols = 0;
+        for (i64 e = 0; e < nnz; ++e) {
+            if (elist[e] < 0) throw std::runtime_error("csr_locality_order: negative column");
+            cols = std::max(cols, elist[e] + 1);
+        }
+        std::vector<i64> cstart((size_t)cols + 1, 0);
+        for (i64 e = 0; e < nnz; ++e) ++cstart[elist[e] + 1];
+        for (i64 c = 0; c < cols; ++c) cstart[c + 1] += cstart[c];
+        std::vector<int32_t> crow((size_t)nnz);
+        {
+            std::vector<i64> fill(cstart.begin(), cstart.end() - 1);
+            for (i64 r = 0; r < rows; ++r)
+                for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) crow[fill[elist[e]]++] = (int32_t)r;
+        }
+        // the closest relative of every row
+        std::vector<int32_t> best((size_t)rows, -1), shared((size_t)rows, 0);
+#pragma omp parallel
+        {
+            std::vector<int32_t> count((size_t)rows, 0), touched;
+#pragma omp for schedule(dynamic, 1024)
+            for (i64 r = 0; r < rows; ++r) {
+                touched.clear();
+                for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) {
+                    const i64 c = elist[e];
+                    if (cstart[c + 1] - cstart[c] > kLocalityHubRows) continue;
+                    for (i64 q = cstart[c]; q < cstart[c + 1]; ++q) {
+                        const int32_t o = crow[q];
+                        if (o != r && count[o]++ == 0) touched.push_back(o);
+                    }
+                }
+                int32_t b = -1, most = 0;
+                for (int32_t o : touched) {
+                    if (count[o] > most || (count[o] == most && o < b)) most = count[o], b = o;
+                    count[o] = 0;
+                }
+                best[r] = b;
+                shared[r] = most;
+            }
+        }
+        // ties that close no cycle, in row order
+        std::vector<int32_t> root((size_t)rows);
+        std::iota(root.begin(), root.end(), 0);
+        auto find = [&](int32_t x) {
+            while (root[x] != x) {
+                root[x] = root[root[x]];
+                x = root[x];
+            }
+            return x;
+        };
+        std::vector<char> kept((size_t)rows, 0);
+        std::vector<i64> astart((size_t)rows + 1, 0);
+        for (i64 r = 0; r < rows; ++r) {
+            if (best[r] < 0) continue;
+            const int32_t a = find((int32_t)r), c = find(best[r]);
+            if (a == c) continue;
+            root[a] = c;
+            kept[r] = 1;
+            ++astart[r + 1];
+            ++astart[best[r] + 1];
+        }
+        for (i64 r = 0; r < rows; ++r) astart[r + 1] += astart[r];
+        struct Tie {
+            int32_t shared, row;
+        };
+        std::vector<Tie> adj((size_t)astart[rows]);
+        {
+            std::vector<i64> fill(astart.begin(), astart.end() - 1);
+            for (i64 r = 0; r < rows; ++r)
+                if (kept[r]) {
+                    adj[fill[r]++] = Tie{shared[r], best[r]};
+                    adj[fill[best[r]]++] = Tie{shared[r], (int32_t)r};
+                }
+        }
+#pragma omp parallel for schedule(dynamic, 4096)
+        for (i64 r = 0; r < rows; ++r)
+            std::sort(adj.begin() + astart[r], adj.begin() + astart[r + 1], [](const Tie &x, const Tie &y) {
+                return x.shared != y.shared ? x.shared > y.shared : x.row < y.row;
+            });
+        // depth-first walk
+        std::vector<int32_t> order;
+        order.reserve((size_t)rows);
+        std::vector<char> seen((size_t)rows, 0);
+        std::vector<i64> next(astart.begin(), astart.end() - 1);
+        std::vector<int32_t> stack;
+        for (i64 i = 0; i < rows; ++i) {
+            if (seen[lex[i]]) continue;
+            seen[lex[i]] = 1;
+            order.push_back(lex[i]);
+            stack.push_back(lex[i]);
+            while (!stack.empty()) {
+                const int32_t top = stack.back();
+                if (next[top] == astart[top + 1]) {
+                    stack.pop_back();
+                    continue;
+                }
+                const int32_t o = adj[next[top]++].row;
+                if (seen[o]) continue;
+                seen[o] = 1;
+                order.push_back(o);
+                stack.push_back(o);
+            }
+        }
         auto *out = new cgnn_arrays;
         out->add(std::move(order));
         return out;

@@ -116,14 +116,17 @@ __device__ __forceinline__ void feature_offsets(int64_t F, int lane, int64_t fof
     }
 }
 
-// Accumulators of one output row: one set, or two in MODE_DUAL (separate members, so
-// that both stay in registers).
+// Accumulator of one output row.  MODE_DUAL keeps the sums over the two sources apart: the
+// entries of a row are sorted by column, so those of the first source come first; when the
+// first entry of the second source arrives the running sum is put aside and started anew.
 template <typename T, int VEC, int TILES, int MODE>
 struct Acc {
-    Pack<T, VEC> a0[TILES];
-    Pack<T, VEC> a1[MODE == MODE_DUAL ? TILES : 1];
+    Pack<T, VEC> a0[TILES];                          // running sum
+    Pack<T, VEC> a1[MODE == MODE_DUAL ? TILES : 1];  // MODE_DUAL: finished sum over the first source
+    bool second_source;                              // MODE_DUAL: a1 is in use
 
     __device__ __forceinline__ void clear() {
+        second_source = false;
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
 #pragma unroll
@@ -135,33 +138,38 @@ struct Acc {
     // entry with gathered tiles x, value w, from source `src` (0 or 1)
     __device__ __forceinline__ void add(const Pack<T, VEC> x[TILES], T w, int src) {
         if constexpr (MODE == MODE_DUAL) {
-            // Both updates are formed and one is kept by a value select.  A branch on
-            // `src` would be turned into an indexed access to the two accumulator sets,
-            // which moves them out of registers into scratch memory.
-            const bool second = src != 0;
+            // At most once per row, so the whole wave jumps over it nearly always.  Written
+            // with value selects under a wave-uniform branch: a branch per lane would be
+            // turned into selects on every entry.
+            const bool change = src != 0 && !second_source;
+            if (__ballot(change)) {
 #pragma unroll
-            for (int t = 0; t < TILES; ++t)
+                for (int t = 0; t < TILES; ++t)
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) {
-                    const T p = x[t].v[i] * w;
-                    const T u0 = a0[t].v[i] + p, u1 = a1[t].v[i] + p;
-                    a0[t].v[i] = second ? a0[t].v[i] : u0;
-                    a1[t].v[i] = second ? u1 : a1[t].v[i];
-                }
-        } else {
-#pragma unroll
-            for (int t = 0; t < TILES; ++t)
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) {
-                    if constexpr (MODE == MODE_VAL) a0[t].v[i] = a0[t].v[i] + x[t].v[i] * w;
-                    else a0[t].v[i] = a0[t].v[i] + x[t].v[i];
-                }
+                    for (int i = 0; i < VEC; ++i) {
+                        a1[t].v[i] = change ? a0[t].v[i] : a1[t].v[i];
+                        a0[t].v[i] = change ? T(0) : a0[t].v[i];
+                    }
+                second_source = second_source || change;
+            }
         }
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) a0[t].v[i] = a0[t].v[i] + x[t].v[i] * w;
+                else a0[t].v[i] = a0[t].v[i] + x[t].v[i];
+            }
     }
     // the row's value on top of `base`: (base + sum1) + sum0 in MODE_DUAL, base + sum otherwise
     __device__ __forceinline__ T total(T base, int t, int i) const {
-        if constexpr (MODE == MODE_DUAL) return (base + a1[t].v[i]) + a0[t].v[i];
-        else return base + a0[t].v[i];
+        if constexpr (MODE == MODE_DUAL) {
+            const T sum0 = second_source ? a1[t].v[i] : a0[t].v[i];
+            const T sum1 = second_source ? a0[t].v[i] : T(0);
+            return (base + sum1) + sum0;
+        } else {
+            return base + a0[t].v[i];
+        }
     }
 };
 

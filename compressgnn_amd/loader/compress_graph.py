@@ -6,8 +6,8 @@ loader/compress_graph.py:6-57; on a GPU it additionally carries the propagation 
 import _paths  # noqa: F401
 import torch
 
-from compressgnn_offline import (csr_hstack, csr_locality_order, csr_permute_rows, csr_row_stats, gen_degree,
-                                 hybird_partition, topo_partition)
+from compressgnn_offline import (csr_hstack, csr_locality_order, csr_permute_rows, gen_degree, hybird_partition,
+                                 topo_partition)
 from sparse_csr import SparseCSR
 
 
@@ -84,20 +84,17 @@ class CompressGraph():
             V, R = self.vertex_cnt, self.rule_cnt
             host = lambda triple: tuple(t.cpu().numpy() for t in triple)
             t = torch.from_numpy
-            rp, ci, val = csr_hstack(host(self.v2v_graph.csr()), host(self.v2r_graph.csr()), V)
-            plan.vertex_stage = rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev, seg)
-            rp, ci, val = csr_hstack(host(self.v2v_graph.csc()), host(self.r2v_graph.csc()), V)
-            # The backward vertex stage runs the row schedule (out-lists are short and even).
-            # Its rows are stored sorted by their column lists, so that rows which gather the
-            # same rows of the gradient are processed together, on one XCD; results do not
-            # depend on the order.
-            longest, _ = csr_row_stats(rp)
-            mean = len(ci) / max(V, 1)
-            if longest <= 8 * max(8.0, mean):  # the rule by which the kernels pick the row schedule
+            # Both vertex stages store their rows in a locality order (rows that gather the same
+            # rows of the input follow each other and are processed on one XCD), which cuts
+            # the misses in the per-XCD L2 caches; results do not depend on the order in the
+            # row schedule, and in the nnz schedule only where a long row is cut into runs.
+            def stage(triple):
+                rp, ci, val = triple
                 order = csr_locality_order(rp, ci)
                 rp, ci, val = csr_permute_rows(rp, ci, val, order)
-                plan.vertex_stage_t = rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev, seg, t(order))
-            else:
-                plan.vertex_stage_t = rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev, seg)
+                return rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev, seg, t(order))
+
+            plan.vertex_stage = stage(csr_hstack(host(self.v2v_graph.csr()), host(self.v2r_graph.csr()), V))
+            plan.vertex_stage_t = stage(csr_hstack(host(self.v2v_graph.csc()), host(self.r2v_graph.csc()), V))
             self._plan = plan
         return self._plan

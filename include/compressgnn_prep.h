@@ -117,9 +117,11 @@ cgnn_arrays *cgnn_csr_hstack(int64_t rows, const int64_t *vlist0, const int64_t 
                              const int64_t *vlist1, const int64_t *elist1, const float *value1,
                              int64_t col_offset);
 
-/* A row order for locality: rows sorted lexicographically by their column lists, so that
- * rows which gather the same columns are neighbours.  -> [order (int32, rows)]: position g
- * of the order holds row order[g]. */
+/* A row order for locality: rows that share many columns follow each other (a depth-first
+ * walk of the forest that ties every row to the row it shares most columns with; trees and
+ * unrelated rows in the lexicographic order of their column lists).  The order depends on
+ * the matrix only, not on the number of threads.  -> [order (int32, rows)]: position g of
+ * the order holds row order[g]. */
 cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const int64_t *elist);
 
 /* The CSR with its rows rearranged: row g of the result is row order[g] of the input

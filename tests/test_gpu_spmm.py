@@ -193,8 +193,8 @@ def test_spmm_f64():
 @pytest.mark.parametrize("F", [16, 128, 200])
 def test_spmm_stored_row_order(rows, F):
     """A block whose rows are stored in another order (rowmap) gives the same bits as the
-    plain block, fresh, accumulating and in the two-source form; the locality order of the
-    host library is a permutation that sorts the rows by their column lists."""
+    plain block, fresh, accumulating and in the two-source form, for the locality order of
+    the host library and for a random permutation."""
     from compressgnn_amd import compressgnn_offline as off
     rng = np.random.default_rng(rows + F)
     cols = 300
@@ -202,8 +202,6 @@ def test_spmm_stored_row_order(rows, F):
     x = rng.standard_normal((cols, F)).astype(np.float32)
     order = off.csr_locality_order(vlist, elist)
     assert sorted(order.tolist()) == list(range(rows))
-    keys = [tuple(elist[vlist[r]:vlist[r + 1]]) for r in order]
-    assert keys == sorted(keys)
     for perm in (order, rng.permutation(rows).astype(np.int32)):
         pv, pe, pw = off.csr_permute_rows(vlist, elist, value, perm)
         plain = abi.DeviceCsr.from_host(rows, cols, vlist, elist, value, DEV)

@@ -222,3 +222,98 @@ def test_row_stats_and_hstack():
     a1 = (np.array([0, 0, 2, 2]), np.array([1, 0]), np.array([4., 5.], np.float32))
     rp, ci, val = off.csr_hstack(a0, a1, 10)
     assert rp.tolist() == [0, 1, 3, 5] and ci.tolist() == [2, 11, 10, 0, 1] and val.tolist() == [1, 4, 5, 2, 3]
+
+
+def _locality_order_by_hand(vlist, elist, hub_rows=256):
+    """The locality order, restated with plain Python loops: every row is tied to the row it
+    shares most columns with (columns listed by more than hub_rows rows do not count; ties
+    go to the lower row), ties that close no cycle are kept in row order, and the forest is
+    walked depth first, closest relatives first, trees in the lexicographic order of the
+    column lists."""
+    rows = len(vlist) - 1
+    lists = [list(elist[vlist[r]:vlist[r + 1]]) for r in range(rows)]
+    users = {}
+    for r, cols in enumerate(lists):
+        for c in cols:
+            users.setdefault(c, []).append(r)
+    best, shared = [-1] * rows, [0] * rows
+    for r, cols in enumerate(lists):
+        count = Counter()
+        for c in cols:
+            if len(users[c]) <= hub_rows:
+                for o in users[c]:
+                    if o != r:
+                        count[o] += 1
+        for o in sorted(count):
+            if count[o] > shared[r]:
+                best[r], shared[r] = o, count[o]
+    root = list(range(rows))
+
+    def find(x):
+        while root[x] != x:
+            x = root[x]
+        return x
+
+    adj = [[] for _ in range(rows)]
+    for r in range(rows):
+        if best[r] >= 0 and find(r) != find(best[r]):
+            root[find(r)] = find(best[r])
+            adj[r].append((-shared[r], best[r]))
+            adj[best[r]].append((-shared[r], r))
+    order, seen = [], [False] * rows
+    for start in sorted(range(rows), key=lambda r: (lists[r], r)):
+        if seen[start]:
+            continue
+        stack = [start]
+        seen[start] = True
+        order.append(start)
+        while stack:
+            for _, o in sorted(adj[stack[-1]]):
+                if not seen[o]:
+                    seen[o] = True
+                    order.append(o)
+                    stack.append(o)
+                    break
+            else:
+                stack.pop()
+    return order
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_locality_order_matches_restatement(seed):
+    rng = np.random.default_rng(seed)
+    rows, cols = [(40, 12), (300, 60), (500, 2000), (700, 90)][seed]
+    lens = rng.integers(0, 9, size=rows)
+    if seed == 3:
+        lens[::7] = 0
+    vlist = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    elist = np.concatenate([np.sort(rng.choice(cols, size=n, replace=False)) for n in lens] + [np.zeros(0, np.int64)])
+    elist = elist.astype(np.int64)
+    if seed == 1:  # a column that more than 256 rows list must not tie rows together
+        keep = [np.union1d(elist[vlist[r]:vlist[r + 1]], [0]) for r in range(rows)]
+        vlist = np.concatenate([[0], np.cumsum([len(k) for k in keep])]).astype(np.int64)
+        elist = np.concatenate(keep).astype(np.int64)
+    got = off.csr_locality_order(vlist, elist)
+    assert got.dtype == np.int32 and sorted(got.tolist()) == list(range(rows))
+    assert got.tolist() == _locality_order_by_hand(vlist, elist)
+    assert off.csr_locality_order(vlist, elist).tolist() == got.tolist()
+
+
+def test_locality_order_keeps_families_together():
+    """Rows with the same column list follow each other when no other row shares a column
+    with them; rows that share nothing are in the lexicographic order of their lists."""
+    rng = np.random.default_rng(11)
+    families = [np.sort(rng.choice(50, size=6, replace=False)) + 50 * k for k in range(30)]
+    owner = rng.permutation(np.repeat(np.arange(30), 4))
+    lists = [families[k] for k in owner]
+    vlist = np.concatenate([[0], np.cumsum([len(x) for x in lists])]).astype(np.int64)
+    elist = np.concatenate(lists).astype(np.int64)
+    order = off.csr_locality_order(vlist, elist)
+    walked = owner[order]
+    assert all(len(set(walked[i:i + 4])) == 1 for i in range(0, len(walked), 4))
+    firsts = [tuple(families[k]) for k in walked[::4]]
+    assert firsts == sorted(firsts)
+    # unrelated rows: pure lexicographic order, shorter list first on a common prefix
+    vlist = np.array([0, 2, 3, 3, 5, 6], np.int64)
+    elist = np.array([7, 9, 4, 6, 8, 2], np.int64)  # rows: [7,9] [4] [] [6,8] [2]
+    assert off.csr_locality_order(vlist, elist).tolist() == [2, 4, 1, 3, 0]
