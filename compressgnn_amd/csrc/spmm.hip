@@ -34,13 +34,14 @@
 // layer/CompressgnnSPMM.py:56-58), so X and Y carry no __restrict__; a row that is
 // written is never gathered in the same launch (levels only read earlier levels).
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.h"
 
 namespace cgnn {
 namespace {
 
-constexpr int kUnroll = 8;        // gathers in flight per lane and tile
+constexpr int kUnroll = 4;        // gathers in flight per lane and tile
 constexpr int kRowUnroll = 8;     // same for the row schedule (4: 9 % slower on web-graph out-lists, 12: 30 %)
 constexpr int kXcds = 8;          // accelerator dies of an MI355X, each with its own L2
 constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
@@ -212,7 +213,7 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
             c -= a.split;
         }
     }
-    const int64_t off = (int64_t)c * a.F + foff;
+    const int64_t off = (int64_t)c * (int32_t)a.F + foff;  // F < 2^31: one 32 x 32 -> 64 bit multiply
     x = load_pack<T, VEC>(base + off);
     if constexpr (MODE == MODE_RELU_MASK) {
         Pack<T, VEC> m = load_pack<T, VEC>(a.M + off);
@@ -228,14 +229,18 @@ __device__ __forceinline__ int out_row(const SpmmArgs<T> &a, int r) {
     return a.rowmap != nullptr ? a.rowmap[r] : r;
 }
 
-// Workgroups are dealt to the XCDs round robin.  With a locality order the grid is a multiple
-// of kXcds and XCD x takes the x-th contiguous share of the stored rows (or runs), so that
-// neighbours in the order meet in one L2.
+// Workgroups are dealt to the XCDs round robin.  With a locality order, XCD x takes every
+// kXcds-th stretch of kXcdStretch consecutive workgroups' worth of stored rows (or runs):
+// neighbours in the order meet in one L2, and every XCD gets the same mix of the matrix
+// (one contiguous share each would leave the XCD with the least reuse to finish last).
+// The grid is a multiple of kXcds * kXcdStretch.
+constexpr int kXcdStretch = 64;
+
 template <typename T>
 __device__ __forceinline__ int logical_block(const SpmmArgs<T> &a) {
     if (a.rowmap == nullptr) return blockIdx.x;
-    const int share = gridDim.x / kXcds;
-    return (blockIdx.x % kXcds) * share + blockIdx.x / kXcds;
+    const int xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;  // turn: this workgroup's number on its XCD
+    return ((turn / kXcdStretch) * kXcds + xcd) * kXcdStretch + turn % kXcdStretch;
 }
 
 // ---------------------------------------------------------------- row schedule --
@@ -256,25 +261,78 @@ __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
         if (!a.accumulate) write_row<T, VEC, TILES, MODE>(a.Y, a.F, row, foff, acc, 0);
         return;
     }
-    for (int e = e0; e < e1; e += kRowUnroll) {
-        int c[kRowUnroll];
-        T w[kRowUnroll];
-        Pack<T, VEC> x[kRowUnroll][TILES];
+    if constexpr (LPR >= kRowUnroll && sizeof(T) == 4) {
+        // The lanes of the group load one entry each (one coalesced load per array for LPR
+        // entries), and every entry is then handed to all lanes through the LDS crossbar:
+        // no address arithmetic and no memory instruction per entry and lane for the indices.
+        const int group_lane0 = 4 * ((threadIdx.x % kWave) - lane);  // byte address of the group's first lane
+        // lanes beyond the width gather feature 0 again (never stored): no test per gather
+        int64_t fld[TILES];
 #pragma unroll
-        for (int u = 0; u < kRowUnroll; ++u) {
-            const int idx = min(e + u, e1 - 1);
-            c[u] = a.colidx[idx];
-            w[u] = a.val ? a.val[idx] : T(1);
+        for (int t = 0; t < TILES; ++t) fld[t] = foff[t] < 0 ? 0 : foff[t];
+        for (int e = e0; e < e1; e += LPR) {
+            int my_c = 0;
+            T my_w = T(1);
+            if (e + lane < e1) {
+                my_c = a.colidx[e + lane];
+                if (a.val) my_w = a.val[e + lane];
+            }
+            const int cnt = min(e1 - e, LPR);
+            for (int u0 = 0; u0 < cnt; u0 += kRowUnroll) {
+                int c[kRowUnroll];
+                T w[kRowUnroll];
+#pragma unroll
+                for (int u = 0; u < kRowUnroll; ++u) {
+                    const int from = group_lane0 + 4 * (u0 + u);
+                    c[u] = __builtin_amdgcn_ds_bpermute(from, my_c);
+                    w[u] = __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, my_w)));
+                }
+                // Entries of the second source are rare (columns that stand for rules): when the
+                // wave has none in this round, the gathers need no choice of source per lane.
+                bool second = false;
+                if constexpr (MODE == MODE_DUAL) {
+#pragma unroll
+                    for (int u = 0; u < kRowUnroll; ++u) second = second || (u0 + u < cnt && c[u] >= a.split);
+                }
+                auto gather_and_add = [&](auto plain) {
+                    constexpr bool kPlain = decltype(plain)::value;  // every entry from the first source
+                    Pack<T, VEC> x[kRowUnroll][TILES];
+#pragma unroll
+                    for (int u = 0; u < kRowUnroll; ++u)
+                        if (u0 + u < cnt) {  // no gathers behind the row's end: repeated ones still cost issue slots
+#pragma unroll
+                            for (int t = 0; t < TILES; ++t)
+                                x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
+                        }
+#pragma unroll
+                    for (int u = 0; u < kRowUnroll; ++u)
+                        if (u0 + u < cnt) acc.add(x[u], w[u], kPlain ? 0 : c[u] >= a.split);
+                };
+                if (MODE != MODE_DUAL || __ballot(second) == 0) gather_and_add(std::true_type{});
+                else gather_and_add(std::false_type{});
+            }
         }
+    } else {
+        for (int e = e0; e < e1; e += kRowUnroll) {
+            int c[kRowUnroll];
+            T w[kRowUnroll];
+            Pack<T, VEC> x[kRowUnroll][TILES];
 #pragma unroll
-        for (int u = 0; u < kRowUnroll; ++u)
-            if (e + u < e1) {  // no gathers behind the row's end: repeated ones still cost issue slots
-#pragma unroll
-                for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
+            for (int u = 0; u < kRowUnroll; ++u) {
+                const int idx = min(e + u, e1 - 1);
+                c[u] = a.colidx[idx];
+                w[u] = a.val ? a.val[idx] : T(1);
             }
 #pragma unroll
-        for (int u = 0; u < kRowUnroll; ++u)
-            if (e + u < e1) acc.add(x[u], w[u], c[u] >= a.split);
+            for (int u = 0; u < kRowUnroll; ++u)
+                if (e + u < e1) {
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
+                }
+#pragma unroll
+            for (int u = 0; u < kRowUnroll; ++u)
+                if (e + u < e1) acc.add(x[u], w[u], c[u] >= a.split);
+        }
     }
     write_row<T, VEC, TILES, MODE>(a.Y, a.F, row, foff, acc, a.accumulate);
 }
@@ -293,7 +351,7 @@ __device__ __forceinline__ int run_boundary(const SpmmArgs<T> &a, int e) {
 }
 
 template <typename T, int VEC, int LPR, int TILES, int MODE>
-__global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
+__global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spmm_nnz_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
     __shared__ int wg_row[GPB];
     __shared__ Pack<T, VEC> wg_carry[TILES][kBlock];
@@ -315,34 +373,98 @@ __global__ __launch_bounds__(kBlock) void spmm_nnz_kernel(SpmmArgs<T> a) {
     bool continues = false;
     if (active) {
         cur = a.rowidx[e0];
-        for (int e = e0; e < e1; e += kUnroll) {
-            int r[kUnroll], c[kUnroll];
-            T w[kUnroll];
-            Pack<T, VEC> x[kUnroll][TILES];
+        if constexpr (LPR >= kUnroll && sizeof(T) == 4) {
+            // As in the row schedule: the lanes of the group load one entry each, and the
+            // entries reach all lanes through the LDS crossbar.
+            const int group_lane0 = 4 * ((threadIdx.x % kWave) - lane);
+            int64_t fld[TILES];  // lanes beyond the width gather feature 0 again (never stored)
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int idx = min(e + u, e1 - 1);
-                r[u] = a.rowidx[idx];
-                c[u] = a.colidx[idx];
-                if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
-                else w[u] = T(1);
+            for (int t = 0; t < TILES; ++t) fld[t] = foff[t] < 0 ? 0 : foff[t];
+            for (int e = e0; e < e1; e += LPR) {
+                int my_r = 0, my_c = 0;
+                T my_w = T(1);
+                if (e + lane < e1) {
+                    my_r = a.rowidx[e + lane];
+                    my_c = a.colidx[e + lane];
+                    if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) my_w = a.val[e + lane];
+                }
+                const int cnt = min(e1 - e, LPR);
+                for (int u0 = 0; u0 < cnt; u0 += kUnroll) {
+                    int r[kUnroll], c[kUnroll];
+                    T w[kUnroll];
+#pragma unroll
+                    for (int u = 0; u < kUnroll; ++u) {
+                        const int from = group_lane0 + 4 * (u0 + u);
+                        r[u] = __builtin_amdgcn_ds_bpermute(from, my_r);
+                        c[u] = __builtin_amdgcn_ds_bpermute(from, my_c);
+                        if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL)
+                            w[u] = __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, my_w)));
+                        else
+                            w[u] = T(1);
+                    }
+                    bool second = false;
+                    if constexpr (MODE == MODE_DUAL) {
+#pragma unroll
+                        for (int u = 0; u < kUnroll; ++u) second = second || (u0 + u < cnt && c[u] >= a.split);
+                    }
+                    auto gather_and_add = [&](auto plain) {
+                        constexpr bool kPlain = decltype(plain)::value;  // every entry from the first source
+                        Pack<T, VEC> x[kUnroll][TILES];
+#pragma unroll
+                        for (int u = 0; u < kUnroll; ++u)
+                            if (u0 + u < cnt) {
+#pragma unroll
+                                for (int t = 0; t < TILES; ++t)
+                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
+                            }
+#pragma unroll
+                        for (int u = 0; u < kUnroll; ++u) {
+                            if (u0 + u < cnt) {
+                                if (r[u] != cur) {
+                                    // row `cur` ends inside this run: finish it here
+                                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+                                    acc.clear();
+                                    cur = r[u];
+                                }
+                                acc.add(x[u], w[u], kPlain ? 0 : c[u] >= a.split);
+                            }
+                        }
+                    };
+                    if (MODE != MODE_DUAL || __ballot(second) == 0) gather_and_add(std::true_type{});
+                    else gather_and_add(std::false_type{});
+                }
             }
+        } else {
+            for (int e = e0; e < e1; e += kUnroll) {
+                int r[kUnroll], c[kUnroll];
+                T w[kUnroll];
+                Pack<T, VEC> x[kUnroll][TILES];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-                if (e + u < e1) {
-#pragma unroll
-                    for (int t = 0; t < TILES; ++t) x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
+                for (int u = 0; u < kUnroll; ++u) {
+                    const int idx = min(e + u, e1 - 1);
+                    r[u] = a.rowidx[idx];
+                    c[u] = a.colidx[idx];
+                    if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
+                    else w[u] = T(1);
                 }
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                if (e + u < e1) {
-                    if (r[u] != cur) {
-                        // row `cur` ends inside this run: finish it here
-                        write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
-                        acc.clear();
-                        cur = r[u];
+                for (int u = 0; u < kUnroll; ++u)
+                    if (e + u < e1) {
+#pragma unroll
+                        for (int t = 0; t < TILES; ++t)
+                            x[u][t] = gather<T, VEC, MODE>(a, c[u], c[u] >= a.split, foff[t]);
                     }
-                    acc.add(x[u], w[u], c[u] >= a.split);
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    if (e + u < e1) {
+                        if (r[u] != cur) {
+                            // row `cur` ends inside this run: finish it here
+                            write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+                            acc.clear();
+                            cur = r[u];
+                        }
+                        acc.add(x[u], w[u], c[u] >= a.split);
+                    }
                 }
             }
         }
@@ -662,7 +784,7 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
     dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
     if (grid.x == 0) return CGNN_OK;
     if ((kind == KIND_ROW || kind == KIND_NNZ) && a.rowmap != nullptr)
-        grid.x = (unsigned)(ceil_div(grid.x, kXcds) * kXcds);
+        grid.x = (unsigned)(ceil_div(grid.x, kXcds * kXcdStretch) * kXcds * kXcdStretch);
     switch (kind) {
         case KIND_ROW:
             if (mode == MODE_DUAL)
