@@ -7,6 +7,12 @@
 // instruction when VEC*sizeof(T) = 16, i.e. global_load_dwordx4 on every lane).
 // Features beyond LPR*VEC*TILES are covered by blockIdx.y.
 //
+// The entries of a row (column, value, row) are loaded once per lane group, one entry per
+// lane with a coalesced load, and handed to all lanes of the group through the LDS
+// crossbar (ds_bpermute); the gathers of a round are issued together, none behind the end
+// of the row.  Loading every entry in every lane made the kernels bound by vector
+// instruction issue (address arithmetic), not by memory.
+//
 // Two schedules:
 //   * row schedule  -- a lane group per row, entries summed in ascending order; the
 //     result is bit-identical to the sequential CPU sum of the reference
@@ -41,7 +47,8 @@
 namespace cgnn {
 namespace {
 
-constexpr int kUnroll = 4;        // gathers in flight per lane and tile
+constexpr int kUnroll = 4;        // gathers in flight per lane and tile, nnz schedule (with 7 waves per SIMD;
+                                  // 8 in flight with 5 waves measured the same)
 constexpr int kRowUnroll = 8;     // same for the row schedule (4: 9 % slower on web-graph out-lists, 12: 30 %)
 constexpr int kXcds = 8;          // accelerator dies of an MI355X, each with its own L2
 constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
