@@ -19,6 +19,7 @@ EXPORTS = [
     "cgnn_last_error", "cgnn_version",
     "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
+    "cgnn_csr_transpose_workspace_bytes", "cgnn_csr_transpose_device",
     "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_hash", "cgnn_lsh_scan", "cgnn_lsh_finish",
     "cgnn_lsh_group_workspace_bytes", "cgnn_lsh_group",
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
@@ -49,7 +50,8 @@ def lib():
         L.cgnn_last_error.restype = ctypes.c_char_p
         L.cgnn_version.restype = ctypes.c_char_p
         for name in ("cgnn_spmm_workspace_bytes", "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_group_workspace_bytes",
-                     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes"):
+                     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes",
+                     "cgnn_csr_transpose_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
         _lib = L
     return _lib
@@ -206,6 +208,29 @@ def lsh_assign_grouped(x, planes, bits):
                            ptr(active), ptr(ws), ctypes.c_size_t(need), st))
     n, largest = (int(v) for v in active.cpu())
     return ids, counts[:n + 1], n, (offsets[:n + 2], perm, sorted_id, largest)
+
+
+def csr_transpose(rowptr, col, value, cols):
+    """(colptr, row, value) of an int64 CSR block on the GPU: the CSR of its transpose, entries
+    sorted by column, ties in storage order."""
+    dev = rowptr.device
+    rows, nnz = rowptr.numel() - 1, col.numel()
+    L = lib()
+    colptr = torch.empty(cols + 1, dtype=torch.int64, device=dev)
+    row = torch.empty(nnz, dtype=torch.int64, device=dev)
+    tval = None if value is None else torch.empty_like(value)
+    bad = torch.empty(1, dtype=torch.int32, device=dev)
+    need = L.cgnn_csr_transpose_workspace_bytes(i64(nnz))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    null = ctypes.c_void_p(0)
+    check(L.cgnn_csr_transpose_device(
+        i64(rows), i64(cols), i64(nnz), ptr(rowptr), ptr(col) if nnz else null,
+        ctypes.c_int(dtype_code(value.dtype) if value is not None else F32),
+        ptr(value) if (value is not None and nnz) else null, ptr(colptr), ptr(row) if nnz else null,
+        ptr(tval) if (tval is not None and nnz) else null, ptr(bad), ptr(ws), ctypes.c_size_t(need), stream_of(rowptr)))
+    if int(bad.item()) != 0:
+        raise CgnnError("csr_transpose: column out of range [0, %d)" % cols)
+    return colptr, row, tval
 
 
 def cluster_members(ids, groups):

@@ -567,6 +567,44 @@ Tensor cluster_reconstruct_backward(Tensor grad, Tensor index, Tensor output, in
     return out;
 }
 
+// (colptr, row, value) of a block held as int64 tensors on a GPU: the CSR of its transpose,
+// in the order SparseTensor.csc() gives.  The one host read (a flag for columns out of
+// range) comes after the last kernel.
+std::tuple<Tensor, Tensor, c10::optional<Tensor>> csr_transpose(Tensor rowptr, Tensor col, c10::optional<Tensor> value,
+                                                                int64_t cols) {
+    TORCH_CHECK(rowptr.is_cuda() && col.is_cuda(), "csr_transpose: tensors must be on a GPU");
+    TORCH_CHECK(rowptr.scalar_type() == torch::kInt64 && col.scalar_type() == torch::kInt64,
+                "csr_transpose: rowptr and col must be int64");
+    TORCH_CHECK(rowptr.dim() == 1 && col.dim() == 1 && rowptr.numel() >= 1 && cols >= 0, "csr_transpose: bad shapes");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(rowptr.device());
+    const int64_t rows = rowptr.numel() - 1, nnz = col.numel();
+    Tensor rp = rowptr.contiguous(), ci = col.contiguous();
+    Tensor val;
+    int dtype = CGNN_F32;
+    if (value.has_value() && value->defined()) {
+        TORCH_CHECK(value->is_cuda() && value->dim() == 1 && value->numel() == nnz,
+                    "csr_transpose: value must have one entry per non-zero");
+        TORCH_CHECK(value->scalar_type() == torch::kFloat32 || value->scalar_type() == torch::kFloat64,
+                    "csr_transpose: value must be float32 or float64");
+        val = value->contiguous();
+        dtype = dtype_code(val);
+    }
+    Tensor colptr = torch::empty({cols + 1}, rp.options());
+    Tensor row = torch::empty({nnz}, rp.options());
+    Tensor tval = val.defined() ? torch::empty_like(val) : Tensor();
+    Tensor bad = torch::empty({1}, rp.options().dtype(torch::kInt32));
+    const size_t bytes = cgnn_csr_transpose_workspace_bytes(nnz);
+    Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, rp.options().dtype(torch::kUInt8));
+    ok(cgnn_csr_transpose_device(rows, cols, nnz, rp.data_ptr<int64_t>(), nnz ? ci.data_ptr<int64_t>() : nullptr, dtype,
+                                 val.defined() && nnz ? val.data_ptr() : nullptr, colptr.data_ptr<int64_t>(),
+                                 nnz ? row.data_ptr<int64_t>() : nullptr, tval.defined() && nnz ? tval.data_ptr() : nullptr,
+                                 bad.data_ptr<int32_t>(), ws.data_ptr(), bytes, current_stream(rp)),
+       "csr_transpose");
+    TORCH_CHECK(bad.item<int32_t>() == 0, "csr_transpose: column out of range [0, ", cols, ")");
+    if (tval.defined()) return {colptr, row, tval};
+    return {colptr, row, c10::nullopt};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -590,6 +628,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("output"), py::arg("groups"), py::arg("relu"), py::arg("members") = py::none());
     // additions of this build
     m.def("cluster_members", &cluster_members, "member lists (offsets, perm, sorted_id) of the clusters");
+    m.def("csr_transpose", &csr_transpose, "CSR -> CSC of an int64 block on the GPU, SparseTensor.csc() order",
+          py::arg("rowptr"), py::arg("col"), py::arg("value"), py::arg("cols"));
     m.def("version", []() { return std::string(cgnn_version()); });
     py::class_<DeviceCsr, std::shared_ptr<DeviceCsr>>(m, "DeviceCsr")
         .def(py::init([](Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows, int64_t cols,

@@ -40,9 +40,8 @@ class CompressGraph():
 
     def to(self, device):
         device = torch.device(device)
-        if device.type == "cuda":
-            for g in self.blocks():
-                g.csc()  # transposes are built on the host, before the blocks move
+        # the transposes for the backward pass are built where the blocks live: on the GPU
+        # after a move there (plan()), by the host library otherwise
         self.v2v_graph = self.v2v_graph.to(device)
         self.v2r_graph = self.v2r_graph.to(device)
         self.r2v_graph = self.r2v_graph.to(device)

@@ -1,7 +1,9 @@
 """SparseCSR: the small part of torch_sparse.SparseTensor that the CompressGNN loader and
 layers use (reference loader/compress_graph.py:21-35, layer/CompressgnnSPMM.py:22-24,68-70):
 a CSR container with csr(), csc(), to() and sparse_sizes().  csc() orders entries by
-column, then row, ties in storage order -- the order SparseTensor.csc() produces."""
+column, then row, ties in storage order -- the order SparseTensor.csc() produces.  A block
+that lives on a GPU is transposed there (stable radix sort by column); a block on the
+host by the host library.  Both give the same arrays."""
 import _paths  # noqa: F401
 import numpy as np
 import torch
@@ -41,6 +43,15 @@ class SparseCSR:
 
     def csc(self):
         """(colptr, row, value) of the same matrix, i.e. the CSR of its transpose."""
+        if self._csc is None and self.device.type == "cuda":
+            import compressgnn_runtime as rt
+            value = self._value
+            if value is not None and value.dtype not in (torch.float32, torch.float64):
+                value = value.to(torch.float32)
+            colptr, row, tval = rt.csr_transpose(self._rowptr, self._col, value, self._sizes[1])
+            if tval is not None and tval.dtype != self._value.dtype:
+                tval = tval.to(self._value.dtype)
+            self._csc = (colptr, row, tval)
         if self._csc is None:
             dev = self.device
             rp = self._rowptr.cpu().numpy()

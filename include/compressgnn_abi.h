@@ -111,6 +111,20 @@ int cgnn_csr_prepare_i64(int64_t rows, int64_t nnz, const int64_t *rowptr64,
 int cgnn_csr_expand_rows(int64_t rows, int64_t nnz, const int32_t *rowptr,
                          int32_t *rowidx, cgnn_stream_t stream);
 
+/* CSR -> CSC of a block given as int64 tensors on the device, in the order
+ * SparseTensor.csc() gives (layer/CompressgnnSPMM.py:68-70 transposes every block of the
+ * compressed graph that way for the backward pass; loader/compress_graph.py:21-35 relies on
+ * the order): entries sorted by column, ties in storage order.  colptr_out has cols + 1
+ * entries, row_out and val_out nnz; val (dtype CGNN_F32 or CGNN_F64) may be NULL.
+ * *bad_column (device) is set to 1 if a column lies outside [0, cols) and to 0 otherwise;
+ * the outputs are meaningless then.  Same arrays, bit for bit, as cgnn_csr_transpose of
+ * the host library. */
+size_t cgnn_csr_transpose_workspace_bytes(int64_t nnz);
+int cgnn_csr_transpose_device(int64_t rows, int64_t cols, int64_t nnz, const int64_t *rowptr,
+                              const int64_t *col, int dtype, const void *val, int64_t *colptr_out,
+                              int64_t *row_out, void *val_out, int32_t *bad_column,
+                              void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
+
 /* ------------------------------------------------- transformation compression -- */
 
 /* Scratch for cgnn_lsh_scan: bytes needed for 2^bits buckets. */
