@@ -20,6 +20,7 @@ EXPORTS = [
     "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
     "cgnn_csr_transpose_workspace_bytes", "cgnn_csr_transpose_device",
+    "cgnn_compress_batch_workspace_bytes", "cgnn_compress_csr_batch_device",
     "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_hash", "cgnn_lsh_scan", "cgnn_lsh_finish",
     "cgnn_lsh_group_workspace_bytes", "cgnn_lsh_group",
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
@@ -51,7 +52,7 @@ def lib():
         L.cgnn_version.restype = ctypes.c_char_p
         for name in ("cgnn_spmm_workspace_bytes", "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_group_workspace_bytes",
                      "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes",
-                     "cgnn_csr_transpose_workspace_bytes"):
+                     "cgnn_csr_transpose_workspace_bytes", "cgnn_compress_batch_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
         _lib = L
     return _lib

@@ -125,6 +125,21 @@ int cgnn_csr_transpose_device(int64_t rows, int64_t cols, int64_t nnz, const int
                               int64_t *row_out, void *val_out, int32_t *bad_column,
                               void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
 
+/* The batch pair merger on the device: what the reference's optional GPU compressor does
+ * (src/offline/bindings/batch_cuda.cpp:3-9 -> compressgraph::compress_cuda, whose source is
+ * not part of the reference tree; loader/compression_backend.py:24-40 calls it).  vlist
+ * (V + 1 entries) and elist (E entries, columns in [0, V)) are int64 arrays on the device.
+ * Result, the same arrays as cgnn_compress_csr_batch of the host library gives: out_ptr
+ * (capacity V + E/2 + 2) holds the V + R + 1 row starts, out_col (capacity E) the vertex
+ * rows written with vertex and rule ids, followed by the two children of every rule;
+ * host_summary[0] = R, host_summary[1] = entries of out_col.  Offline work: the call waits
+ * for the device (three small reads per round) and returns when the arrays are complete. */
+size_t cgnn_compress_batch_workspace_bytes(int64_t V, int64_t E);
+int cgnn_compress_csr_batch_device(int64_t V, int64_t E, const int64_t *vlist, const int64_t *elist,
+                                   int rounds, int min_pair_frequency, int32_t *out_ptr,
+                                   int32_t *out_col, int64_t *host_summary, void *workspace,
+                                   size_t workspace_bytes, cgnn_stream_t stream);
+
 /* ------------------------------------------------- transformation compression -- */
 
 /* Scratch for cgnn_lsh_scan: bytes needed for 2^bits buckets. */
