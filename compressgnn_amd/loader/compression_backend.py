@@ -1,7 +1,7 @@
 """Backend selection for the batch compressor, with the reference's interface
-(loader/compression_backend.py:6-40).  This build has one compressor (host C++,
-compressgnn_offline.compress_csr_batch); 'auto' resolves to it, 'cuda' reports that no
-GPU compressor is installed."""
+(loader/compression_backend.py:6-40).  Two compressors give the same arrays: the host one
+(compressgnn_offline.compress_csr_batch) and the GPU one (compressgnn_batch_cuda, HIP
+kernels); 'auto' takes the GPU one when a GPU is usable."""
 import _paths  # noqa: F401
 import importlib
 import operator
