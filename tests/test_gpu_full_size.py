@@ -1,0 +1,111 @@
+"""The benchmark configurations at their full sizes, checked through properties that do not
+need a second implementation at that size: the compressed propagation of the 325,557-vertex
+graph against the plain A^T x of the same graph (float64 on the host), its backward pass
+through the adjoint identity <A x, g> = <x, A^T g> and against the forward of the reversed
+graph, reproducibility bit for bit; the 2,449,029-node cluster path through sums that every
+exact implementation preserves (counts add up to N, count-weighted representatives add up to
+the column sums, reconstruct returns the representative of every node's cluster, gradients
+are adjoint)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path[:0] = [ROOT, os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compressgnn_amd", "layer"),
+                os.path.join(ROOT, "compressgnn_amd", "loader")]
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def test_propagation_at_full_size():
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    from KPropagate import KPropagate
+    V, F = 325557, 128
+    v, e = off.gen_copy_model(V, 9.8, 0.7, 1)
+    rng = np.random.default_rng(12)
+    x_np = rng.standard_normal((V, F)).astype(np.float32)
+    g_np = rng.standard_normal((V, F)).astype(np.float32)
+    mask = np.zeros(V, dtype=bool)
+    data = CompressgnnData(x_np, (v, e), np.zeros(V, np.int64), mask, mask, mask, add_self_loop=True,
+                           normalize=True, graph_type="csr", verbose=False)
+    assert data.rule_cnt > 0
+    data.to(DEV)
+    x = data.x.clone().requires_grad_(True)
+    prop = KPropagate()
+    out = prop(x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    g = torch.from_numpy(g_np).to(DEV)
+    (gx,) = torch.autograd.grad(out, x, g)
+    out_np, gx_np = out.detach().cpu().numpy(), gx.cpu().numpy()
+    # forward = A_hat^T x of the uncompressed graph (float64, host), fp32 tolerance of the task
+    v2, e2 = off.add_self_loop_csr(v, e)
+    d = off.get_norm_degree(e2, V).astype(np.float64)
+    src = np.repeat(np.arange(V), np.diff(v2))
+    w = d[src] * d[e2]
+    import scipy.sparse as sp
+    A = sp.csr_matrix((w, e2, v2), shape=(V, V))  # A[s, d]
+    want = A.T @ x_np.astype(np.float64)
+    assert np.all(np.abs(out_np - want) <= 1e-5 * np.abs(want) + 1e-6)
+    # backward = A_hat g, and the adjoint identity ties the two passes together
+    want_g = A @ g_np.astype(np.float64)
+    assert np.all(np.abs(gx_np - want_g) <= 1e-5 * np.abs(want_g) + 1e-6)
+    lhs = float((out_np.astype(np.float64) * g_np).sum())
+    rhs = float((x_np.astype(np.float64) * gx_np).sum())
+    assert abs(lhs - rhs) <= 1e-6 * max(1.0, abs(lhs))
+    # same bits run to run, and linear: P(2x) = 2 P(x) exactly (scaling by two is exact)
+    again = prop(data.x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    assert torch.equal(again, out.detach())
+    twice = prop(2 * data.x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    assert torch.equal(twice, 2 * out.detach())
+
+
+def test_cluster_path_at_full_size():
+    import compressgnn_runtime as rt
+    N, F, H, F2 = 2449029, 100, 16, 256
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(5)
+    centres = 2.0 * torch.randn(47, F, device=DEV, generator=gen)
+    which = torch.randint(0, 47, (N,), device=DEV, generator=gen)
+    x = centres[which] + torch.randn(N, F, device=DEV, generator=gen)
+    planes = torch.randn(F, H, device=DEV, generator=gen)
+    ids, counts, active, members = rt.cluster_assign_members(x, planes, H)
+    assert ids.dtype == torch.int64 and counts.dtype == torch.int32 and counts.numel() == active + 1
+    assert int(counts[0]) == 0 and int(counts.sum()) == N and int(counts.min(dim=0).values) >= 0
+    assert int(ids.min()) >= 1 and int(ids.max()) == active
+    assert torch.equal(torch.bincount(ids, minlength=active + 1).to(torch.int32), counts)
+    # equal codes <=> equal ids: ids are the ranks of the sign patterns, MSB first
+    code = ((x.double() @ planes.double()) > 0).long()  # exact enough away from zero; compare only the partition
+    packed = (code * (2 ** torch.arange(H - 1, -1, -1, device=DEV))).sum(1)
+    order = torch.argsort(ids)
+    changes_ids = int((ids[order][1:] != ids[order][:-1]).sum())
+    assert changes_ids == active - 1
+    disagree = int(((packed[order][1:] != packed[order][:-1]) != (ids[order][1:] != ids[order][:-1])).sum())
+    assert disagree <= 64  # rows whose fp32 projection is within rounding of zero may change sides in float64
+    reps = rt.cluster_mean(x, ids, counts, members)
+    # count-weighted representatives add up to the column sums (float64 reference sum)
+    total = (reps.double() * counts.double()[:, None]).sum(0)
+    want = x.double().sum(0)
+    assert torch.all((total - want).abs() <= 1e-5 * x.double().abs().sum(0))
+    assert torch.equal(reps[0], torch.zeros(F, device=DEV))
+    # reconstruct: every node gets its cluster's row (+ bias, ReLU)
+    W = torch.randn(F2, F, device=DEV, generator=gen) / 10
+    bias = torch.randn(F2, device=DEV, generator=gen)
+    hidden = reps @ W.t()
+    y = rt.cluster_reconstruct(hidden, ids, bias, True, members)
+    probe = torch.randint(0, N, (4096,), device=DEV, generator=gen)
+    assert torch.equal(y[probe], torch.relu(hidden[ids[probe]] + bias))
+    # gradients are the adjoints of the forward maps
+    gy = torch.randn(N, F2, device=DEV, generator=gen)
+    gh = rt.cluster_reconstruct_backward(gy, ids, y, active + 1, True, members)
+    lhs = float(((y > 0) * gy).double().sum(0) @ torch.ones(F2, device=DEV, dtype=torch.double))
+    rhs = float(gh.double().sum())
+    assert abs(lhs - rhs) <= 1e-6 * float(gy.double().abs().sum())
+    gr = torch.randn(active + 1, F, device=DEV, generator=gen)
+    gxm = rt.cluster_mean_backward(gr, ids, counts, members)
+    lhs = float((reps.double() * gr.double()).sum())
+    rhs = float((x.double() * gxm.double()).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(1.0, float((x.double() * gxm.double()).abs().sum()))
