@@ -901,7 +901,10 @@ cgnn_arrays *cgnn_compress_csr_batch(int64_t V, const int64_t *vlist, const int6
 
 // Columns listed by more rows than this are left out when rows are matched by the columns
 // they share: nearly every pair of rows shares such a column (and it stays in cache anyway).
+// The limit is halved until matching costs at most kLocalityWork steps per non-zero
+// (a column listed by d rows costs d * d steps).
 static const i64 kLocalityHubRows = 256;
+static const i64 kLocalityWork = 64;
 
 cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const int64_t *elist) {
     // Rows that gather the same columns should be processed one after the other, so that
@@ -946,6 +949,15 @@ cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const i
             for (i64 r = 0; r < rows; ++r)
                 for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) crow[fill[elist[e]]++] = (int32_t)r;
         }
+        i64 hub_rows = kLocalityHubRows;
+        for (; hub_rows > 2; hub_rows /= 2) {
+            double steps = 0;
+            for (i64 c = 0; c < cols; ++c) {
+                const double d = (double)(cstart[c + 1] - cstart[c]);
+                if (d <= (double)hub_rows) steps += d * d;
+            }
+            if (steps <= (double)kLocalityWork * (double)std::max<i64>(nnz, 1)) break;
+        }
         // the closest relative of every row
         std::vector<int32_t> best((size_t)rows, -1), shared((size_t)rows, 0);
 #pragma omp parallel
@@ -956,7 +968,7 @@ cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const i
                 touched.clear();
                 for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) {
                     const i64 c = elist[e];
-                    if (cstart[c + 1] - cstart[c] > kLocalityHubRows) continue;
+                    if (cstart[c + 1] - cstart[c] > hub_rows) continue;
                     for (i64 q = cstart[c]; q < cstart[c + 1]; ++q) {
                         const int32_t o = crow[q];
                         if (o != r && count[o]++ == 0) touched.push_back(o);

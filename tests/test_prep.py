@@ -224,7 +224,7 @@ def test_row_stats_and_hstack():
     assert rp.tolist() == [0, 1, 3, 5] and ci.tolist() == [2, 11, 10, 0, 1] and val.tolist() == [1, 4, 5, 2, 3]
 
 
-def _locality_order_by_hand(vlist, elist, hub_rows=256):
+def _locality_order_by_hand(vlist, elist, hub_rows=256, work=64):
     """The locality order, restated with plain Python loops: every row is tied to the row it
     shares most columns with (columns listed by more than hub_rows rows do not count; ties
     go to the lower row), ties that close no cycle are kept in row order, and the forest is
@@ -236,6 +236,9 @@ def _locality_order_by_hand(vlist, elist, hub_rows=256):
     for r, cols in enumerate(lists):
         for c in cols:
             users.setdefault(c, []).append(r)
+    nnz = sum(len(x) for x in lists)
+    while hub_rows > 2 and sum(len(u) ** 2 for u in users.values() if len(u) <= hub_rows) > work * max(nnz, 1):
+        hub_rows //= 2
     best, shared = [-1] * rows, [0] * rows
     for r, cols in enumerate(lists):
         count = Counter()
@@ -297,6 +300,20 @@ def test_locality_order_matches_restatement(seed):
     assert got.dtype == np.int32 and sorted(got.tolist()) == list(range(rows))
     assert got.tolist() == _locality_order_by_hand(vlist, elist)
     assert off.csr_locality_order(vlist, elist).tolist() == got.tolist()
+
+
+def test_locality_order_limits_its_work():
+    """100 rows that all list the same 50 columns would cost 100 steps per non-zero to match:
+    the limit on shared columns is halved until those columns no longer count, and the rows
+    (which then share nothing but differ in one private column) come out in lexicographic order."""
+    rng = np.random.default_rng(8)
+    private = rng.permutation(100) + 50
+    lists = [np.concatenate([np.arange(50), [private[r]]]) for r in range(100)]
+    vlist = np.concatenate([[0], np.cumsum([len(x) for x in lists])]).astype(np.int64)
+    elist = np.concatenate(lists).astype(np.int64)
+    got = off.csr_locality_order(vlist, elist).tolist()
+    assert got == _locality_order_by_hand(vlist, elist)
+    assert got == np.argsort(private).tolist()
 
 
 def test_locality_order_keeps_families_together():
