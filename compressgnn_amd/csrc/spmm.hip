@@ -240,8 +240,10 @@ __device__ __forceinline__ int out_row(const SpmmArgs<T> &a, int r) {
 // kXcds-th stretch of kXcdStretch consecutive workgroups' worth of stored rows (or runs):
 // neighbours in the order meet in one L2, and every XCD gets the same mix of the matrix
 // (one contiguous share each would leave the XCD with the least reuse to finish last).
-// The grid is a multiple of kXcds * kXcdStretch.
-constexpr int kXcdStretch = 64;
+// A stretch is about as long as the workgroups an XCD holds at a time, so an XCD works on
+// one region of the order at once (64 and 512 measured 1.5 % slower on the web graph, 1024
+// 20 %: too few stretches to even out).  The grid is a multiple of kXcds * kXcdStretch.
+constexpr int kXcdStretch = 256;
 
 template <typename T>
 __device__ __forceinline__ int logical_block(const SpmmArgs<T> &a) {
