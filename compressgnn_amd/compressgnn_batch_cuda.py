@@ -65,4 +65,8 @@ def compress_csr_batch(vlist, elist, rounds=12, min_pair_frequency=16):
             raise ValueError(msg)
         raise RuntimeError(msg)
     R, n = int(summary[0]), int(summary[1])
-    return out_ptr[:V + R + 1].cpu().numpy(), out_col[:n].cpu().numpy(), V, R
+    result = out_ptr[:V + R + 1].cpu().numpy(), out_col[:n].cpu().numpy(), V, R
+    # the workspace (about 70 bytes per edge) goes back to the device, not into torch's cache
+    del dv, de, out_ptr, out_col, ws
+    torch.cuda.empty_cache()
+    return result
