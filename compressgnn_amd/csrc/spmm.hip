@@ -237,19 +237,26 @@ __device__ __forceinline__ int out_row(const SpmmArgs<T> &a, int r) {
 }
 
 // Workgroups are dealt to the XCDs round robin.  With a locality order, XCD x takes every
-// kXcds-th stretch of kXcdStretch consecutive workgroups' worth of stored rows (or runs):
-// neighbours in the order meet in one L2, and every XCD gets the same mix of the matrix
-// (one contiguous share each would leave the XCD with the least reuse to finish last).
-// A stretch is about as long as the workgroups an XCD holds at a time, so an XCD works on
-// one region of the order at once (64 and 512 measured 1.5 % slower on the web graph, 1024
-// 20 %: too few stretches to even out).  The grid is a multiple of kXcds * kXcdStretch.
-constexpr int kXcdStretch = 256;
+// kXcds-th stretch of consecutive workgroups' worth of stored rows (or runs): neighbours in
+// the order meet in one L2, and every XCD gets the same mix of the matrix (one contiguous
+// share each would leave the XCD with the least reuse to finish last).  A stretch holds
+// kXcdStretchGroups lane groups, about what an XCD holds at a time at F = 128, so an XCD works
+// on one region of the order at once (a quarter and twice that measured 1.5 % slower on the
+// web graph, four times 20 %: too few stretches to even out).  The grid is a multiple of
+// kXcds stretches.
+constexpr int kXcdStretchGroups = 2048;
 
-template <typename T>
+template <int GPB>
+constexpr int xcd_stretch() {
+    return kXcdStretchGroups / GPB > 0 ? kXcdStretchGroups / GPB : 1;
+}
+
+template <int GPB, typename T>
 __device__ __forceinline__ int logical_block(const SpmmArgs<T> &a) {
     if (a.rowmap == nullptr) return blockIdx.x;
+    constexpr int kStretch = xcd_stretch<GPB>();
     const int xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;  // turn: this workgroup's number on its XCD
-    return ((turn / kXcdStretch) * kXcds + xcd) * kXcdStretch + turn % kXcdStretch;
+    return ((turn / kStretch) * kXcds + xcd) * kStretch + turn % kStretch;
 }
 
 // ---------------------------------------------------------------- row schedule --
@@ -257,7 +264,7 @@ template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
     const int lane = threadIdx.x % LPR;
-    int row = logical_block(a) * GPB + threadIdx.x / LPR;
+    int row = logical_block<GPB>(a) * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
     if (row >= a.rows) return;
     const int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
@@ -270,7 +277,8 @@ __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
         if (!a.accumulate) write_row<T, VEC, TILES, MODE>(a.Y, a.F, row, foff, acc, 0);
         return;
     }
-    if constexpr (LPR >= kRowUnroll && sizeof(T) == 4) {
+    if constexpr (sizeof(T) == 4) {
+        constexpr int RU = LPR < kRowUnroll ? LPR : kRowUnroll;  // entries per round: no more than lanes to stage them
         // The lanes of the group load one entry each (one coalesced load per array for LPR
         // entries), and every entry is then handed to all lanes through the LDS crossbar:
         // no address arithmetic and no memory instruction per entry and lane for the indices.
@@ -287,11 +295,11 @@ __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
                 if (a.val) my_w = a.val[e + lane];
             }
             const int cnt = min(e1 - e, LPR);
-            for (int u0 = 0; u0 < cnt; u0 += kRowUnroll) {
-                int c[kRowUnroll];
-                T w[kRowUnroll];
+            for (int u0 = 0; u0 < cnt; u0 += RU) {
+                int c[RU];
+                T w[RU];
 #pragma unroll
-                for (int u = 0; u < kRowUnroll; ++u) {
+                for (int u = 0; u < RU; ++u) {
                     const int from = group_lane0 + 4 * (u0 + u);
                     c[u] = __builtin_amdgcn_ds_bpermute(from, my_c);
                     w[u] = __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, my_w)));
@@ -301,20 +309,20 @@ __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
                 bool second = false;
                 if constexpr (MODE == MODE_DUAL) {
 #pragma unroll
-                    for (int u = 0; u < kRowUnroll; ++u) second = second || (u0 + u < cnt && c[u] >= a.split);
+                    for (int u = 0; u < RU; ++u) second = second || (u0 + u < cnt && c[u] >= a.split);
                 }
                 auto gather_and_add = [&](auto plain) {
                     constexpr bool kPlain = decltype(plain)::value;  // every entry from the first source
-                    Pack<T, VEC> x[kRowUnroll][TILES];
+                    Pack<T, VEC> x[RU][TILES];
 #pragma unroll
-                    for (int u = 0; u < kRowUnroll; ++u)
+                    for (int u = 0; u < RU; ++u)
                         if (u0 + u < cnt) {  // no gathers behind the row's end: repeated ones still cost issue slots
 #pragma unroll
                             for (int t = 0; t < TILES; ++t)
                                 x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
                         }
 #pragma unroll
-                    for (int u = 0; u < kRowUnroll; ++u)
+                    for (int u = 0; u < RU; ++u)
                         if (u0 + u < cnt) acc.add(x[u], w[u], kPlain ? 0 : c[u] >= a.split);
                 };
                 if (MODE != MODE_DUAL || __ballot(second) == 0) gather_and_add(std::true_type{});
@@ -365,7 +373,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     __shared__ int wg_row[GPB];
     __shared__ Pack<T, VEC> wg_carry[TILES][kBlock];
     const int lane = threadIdx.x % LPR, grp = threadIdx.x / LPR;
-    int seg = logical_block(a) * GPB + grp;
+    int seg = logical_block<GPB>(a) * GPB + grp;
     if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
     int e0 = 0, e1 = 0;
     if (seg < a.nseg) {
@@ -793,7 +801,7 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int gr
     dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
     if (grid.x == 0) return CGNN_OK;
     if ((kind == KIND_ROW || kind == KIND_NNZ) && a.rowmap != nullptr)
-        grid.x = (unsigned)(ceil_div(grid.x, kXcds * kXcdStretch) * kXcds * kXcdStretch);
+        grid.x = (unsigned)(ceil_div(grid.x, kXcds * xcd_stretch<GPB>()) * kXcds * xcd_stretch<GPB>());
     switch (kind) {
         case KIND_ROW:
             if (mode == MODE_DUAL)
