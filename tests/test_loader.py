@@ -113,9 +113,14 @@ def test_unsupported_paths_fail_loudly():
 
 def test_backend_resolution():
     import compression_backend as dispatch
-    assert dispatch.resolve_backend('auto') == 'cpu' and dispatch.resolve_backend('cpu') == 'cpu'
-    with pytest.raises(RuntimeError):
-        dispatch.resolve_backend('cuda')
+    import torch
+    assert dispatch.resolve_backend('cpu') == 'cpu'
+    if torch.cuda.is_available():  # the GPU compressor is picked where a GPU is usable
+        assert dispatch.resolve_backend('auto') == 'cuda' and dispatch.resolve_backend('cuda') == 'cuda'
+    else:
+        assert dispatch.resolve_backend('auto') == 'cpu'
+        with pytest.raises(RuntimeError):
+            dispatch.resolve_backend('cuda')
     for bad in ['wrong', 'legacy', None]:
         with pytest.raises(ValueError):
             dispatch.resolve_backend(bad)
