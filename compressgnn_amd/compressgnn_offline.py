@@ -21,7 +21,7 @@ EXPORTS = [
     "cgnn_filter_csr", "cgnn_depth_filter_csr", "cgnn_gen_vertex_order_csr", "cgnn_gen_vertex_order_csc",
     "cgnn_compress_csr_batch", "cgnn_csr_hstack", "cgnn_csr_row_stats", "cgnn_gen_chung_lu", "cgnn_gen_copy_model",
     "cgnn_add_self_loop_coo", "cgnn_gcn_norm_coo_compress", "cgnn_gen_edge_order",
-    "cgnn_csr_locality_order", "cgnn_csr_permute_rows",
+    "cgnn_csr_locality_order", "cgnn_csr_permute_rows", "cgnn_csr_fold_levels",
 ]
 
 _NP_TYPES = {0: np.int64, 1: np.float32, 2: np.int32}
@@ -262,6 +262,20 @@ def csr_hstack(a0, a1, col_offset):
     (v, e, w), _ = _take(lib().cgnn_csr_hstack(ctypes.c_int64(len(v0) - 1), _p(v0), _p(e0), _p(w0), _p(v1), _p(e1),
                                                _p(w1), ctypes.c_int64(col_offset)))
     return v, e, w
+
+
+def csr_fold_levels(base, levels):
+    """The CSR triple `base` (R rows) after the in-place updates base[r] += sum_c L[r, c] * base[c]
+    for every level L (a list of R x R CSR triples, applied in order), as one matrix."""
+    v, e, w = _i64(base[0]), _i64(base[1]), _f32(base[2])
+    lv = [_i64(l[0]) for l in levels]
+    le = [_i64(l[1]) for l in levels]
+    lw = [_f32(l[2]) for l in levels]
+    n = len(levels)
+    ptrs = lambda arrs: (ctypes.c_void_p * max(n, 1))(*[a.ctypes.data for a in arrs])
+    (nv, ne, nw), _ = _take(lib().cgnn_csr_fold_levels(ctypes.c_int64(len(v) - 1), _p(v), _p(e), _p(w), ctypes.c_int(n),
+                                                     ptrs(lv), ptrs(le), ptrs(lw)))
+    return nv, ne, nw
 
 
 def csr_locality_order(vlist, elist):

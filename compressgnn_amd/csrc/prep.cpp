@@ -1052,6 +1052,63 @@ cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const i
     });
 }
 
+cgnn_arrays *cgnn_csr_fold_levels(int64_t R, const int64_t *vlist, const int64_t *elist, const float *value,
+                                  int levels, const int64_t *const *level_vlists,
+                                  const int64_t *const *level_elists, const float *const *level_values) {
+    // B (R rows) followed by the in-place updates B[r] += sum_c L_k[r, c] * B[c] for k = 0,
+    // 1, ... (the rule levels of the compressed propagation, layer/CompressgnnSPMM.py:56-58 of
+    // the reference), as one matrix: row r of the result is the row after all updates, its
+    // entries merged by column in ascending order.  A level only reads rows that it does not
+    // write, so the rows can be rewritten one after the other.
+    if (R < 0 || !vlist || levels < 0 || (levels > 0 && (!level_vlists || !level_elists))) {
+        set_error("csr_fold_levels: bad arguments");
+        return nullptr;
+    }
+    return guarded([&] {
+        typedef std::pair<i64, float> Entry;
+        std::vector<std::vector<Entry>> rows((size_t)R);
+        for (i64 r = 0; r < R; ++r)
+            for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) rows[r].emplace_back(elist[e], value ? value[e] : 1.0f);
+        std::vector<Entry> acc;
+        for (int k = 0; k < levels; ++k) {
+            const i64 *lv = level_vlists[k], *le = level_elists[k];
+            const float *lw = level_values ? level_values[k] : nullptr;
+            for (i64 r = 0; r < R; ++r) {
+                if (lv[r] == lv[r + 1]) continue;
+                acc = rows[r];
+                for (i64 e = lv[r]; e < lv[r + 1]; ++e) {
+                    const i64 c = le[e];
+                    if (c < 0 || c >= R) throw std::runtime_error("csr_fold_levels: level column out of range");
+                    if (lv[c] != lv[c + 1]) throw std::runtime_error("csr_fold_levels: a level reads a row that it writes");
+                    const float w = lw ? lw[e] : 1.0f;
+                    for (const Entry &x : rows[c]) acc.emplace_back(x.first, w * x.second);
+                }
+                std::stable_sort(acc.begin(), acc.end(), [](const Entry &a, const Entry &b) { return a.first < b.first; });
+                std::vector<Entry> merged;
+                for (const Entry &x : acc) {
+                    if (!merged.empty() && merged.back().first == x.first) merged.back().second += x.second;
+                    else merged.push_back(x);
+                }
+                rows[r].swap(merged);
+            }
+        }
+        std::vector<i64> nv((size_t)R + 1, 0), ne;
+        std::vector<float> nw;
+        for (i64 r = 0; r < R; ++r) {
+            nv[r + 1] = nv[r] + (i64)rows[r].size();
+            for (const Entry &x : rows[r]) {
+                ne.push_back(x.first);
+                nw.push_back(x.second);
+            }
+        }
+        auto *out = new cgnn_arrays;
+        out->add(std::move(nv));
+        out->add(std::move(ne));
+        out->add(std::move(nw));
+        return out;
+    });
+}
+
 cgnn_arrays *cgnn_csr_permute_rows(int64_t rows, const int64_t *vlist, const int64_t *elist, const float *value,
                                    const int32_t *order) {
     if (rows < 0 || !vlist || (rows > 0 && !order)) {

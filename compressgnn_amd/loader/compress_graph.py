@@ -6,8 +6,8 @@ loader/compress_graph.py:6-57; on a GPU it additionally carries the propagation 
 import _paths  # noqa: F401
 import torch
 
-from compressgnn_offline import (csr_hstack, csr_locality_order, csr_permute_rows, gen_degree, hybird_partition,
-                                 topo_partition)
+from compressgnn_offline import (csr_fold_levels, csr_hstack, csr_locality_order, csr_permute_rows, gen_degree,
+                                 hybird_partition, topo_partition)
 from sparse_csr import SparseCSR
 
 
@@ -30,6 +30,11 @@ class CompressGraph():
                                                 [lv[0] for lv in r2r_list], [lv[1] for lv in r2r_list])
         self.vertex_degree = t(vertex_degree)
         self.rule_degree = t(rule_degree)
+        # The rule levels are folded into the rule stage when the device plan is built: the
+        # rules then aggregate all the vertices they stand for in one launch, forward and
+        # backward, instead of one more launch per level (the same sums in another order).
+        # Set to False before plan() for the launch-per-level form of the reference.
+        self.fold_levels = True
         self._plan = None
 
     def __repr__(self):
@@ -76,13 +81,24 @@ class CompressGraph():
                 cp, row, val = g.csc()
                 return rt.DeviceCsr(cp, row, val, g.sparse_size(1), g.sparse_size(0), dev, seg)
 
-            plan = rt.PropagationPlan(
-                fwd(self.v2v_graph), fwd(self.v2r_graph), fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
-                bwd(self.v2v_graph), bwd(self.v2r_graph), bwd(self.r2v_graph), [bwd(g) for g in self.r2r_graph])
-            # the vertex stage reads [v2v | v2r] (forward) and [v2v^T | r2v^T] (backward) in one pass
             V, R = self.vertex_cnt, self.rule_cnt
             host = lambda triple: tuple(t.cpu().numpy() for t in triple)
             t = torch.from_numpy
+            if getattr(self, "fold_levels", True) and self.step > 0:
+                # forward: rule_out = (I + L_last) ... (I + L_0) r2v x; backward, with the
+                # transposed levels in reverse order: rule_g = (I + L_0^T) ... (I + L_last^T) v2r^T g
+                rp, ci, val = csr_fold_levels(host(self.r2v_graph.csr()), [host(g.csr()) for g in self.r2r_graph])
+                rules_fwd = rt.DeviceCsr(t(rp), t(ci), t(val), R, V, dev, seg)
+                rp, ci, val = csr_fold_levels(host(self.v2r_graph.csc()),
+                                              [host(g.csc()) for g in reversed(self.r2r_graph)])
+                rules_bwd = rt.DeviceCsr(t(rp), t(ci), t(val), R, V, dev, seg)
+                plan = rt.PropagationPlan(fwd(self.v2v_graph), fwd(self.v2r_graph), rules_fwd, [],
+                                          bwd(self.v2v_graph), rules_bwd, bwd(self.r2v_graph), [])
+            else:
+                plan = rt.PropagationPlan(
+                    fwd(self.v2v_graph), fwd(self.v2r_graph), fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
+                    bwd(self.v2v_graph), bwd(self.v2r_graph), bwd(self.r2v_graph), [bwd(g) for g in self.r2r_graph])
+            # the vertex stage reads [v2v | v2r] (forward) and [v2v^T | r2v^T] (backward) in one pass
             # Both vertex stages store their rows in a locality order (rows that gather the same
             # rows of the input follow each other and are processed on one XCD), which cuts
             # the misses in the per-XCD L2 caches; results do not depend on the order in the

@@ -124,6 +124,14 @@ cgnn_arrays *cgnn_csr_hstack(int64_t rows, const int64_t *vlist0, const int64_t 
  * the order holds row order[g]. */
 cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const int64_t *elist);
 
+/* A block B (R rows) with the rule levels folded in: the result of the in-place updates
+ * B[r] += sum_c L_k[r, c] * B[c], k = 0 .. levels-1 (layer/CompressgnnSPMM.py:56-58 applies
+ * them as one product per level), as one matrix with the entries of a row merged by column.
+ * Every level matrix is R x R and reads only rows it does not write.  -> [vlist, elist, value] */
+cgnn_arrays *cgnn_csr_fold_levels(int64_t R, const int64_t *vlist, const int64_t *elist, const float *value,
+                                  int levels, const int64_t *const *level_vlists,
+                                  const int64_t *const *level_elists, const float *const *level_values);
+
 /* The CSR with its rows rearranged: row g of the result is row order[g] of the input
  * (value may be NULL).  -> [vlist, elist, value] */
 cgnn_arrays *cgnn_csr_permute_rows(int64_t rows, const int64_t *vlist, const int64_t *elist,

@@ -334,3 +334,42 @@ def test_locality_order_keeps_families_together():
     vlist = np.array([0, 2, 3, 3, 5, 6], np.int64)
     elist = np.array([7, 9, 4, 6, 8, 2], np.int64)  # rows: [7,9] [4] [] [6,8] [2]
     assert off.csr_locality_order(vlist, elist).tolist() == [2, 4, 1, 3, 0]
+
+
+def test_fold_levels_equals_the_level_by_level_updates():
+    """csr_fold_levels against the dense in-place updates B[r] += sum_c L_k[r, c] B[c], on
+    levels shaped like topo_partition's (a level reads only rows it does not write)."""
+    rng = np.random.default_rng(21)
+    R, Vn = 60, 40
+    dense = np.where(rng.random((R, Vn)) < 0.15, rng.standard_normal((R, Vn)), 0.0).astype(np.float32)
+
+    def to_csr(m):
+        rp = np.concatenate([[0], np.cumsum((m != 0).sum(1))]).astype(np.int64)
+        rows, cols = np.nonzero(m)
+        return rp, cols.astype(np.int64), m[rows, cols].astype(np.float32)
+
+    # level k writes rows [20k + 20, 20k + 40) and reads rows below 20k + 20
+    levels, want = [], dense.astype(np.float64)
+    for k in range(2):
+        L = np.zeros((R, R), np.float32)
+        lo, hi = 20 * k + 20, 20 * k + 40
+        block = np.where(rng.random((hi - lo, lo)) < 0.2, rng.integers(1, 3, (hi - lo, lo)), 0)
+        L[lo:hi, :lo] = block
+        levels.append(to_csr(L))
+        want = want + L.astype(np.float64) @ want
+    rp, ci, val = off.csr_fold_levels(to_csr(dense), levels)
+    got = np.zeros((R, Vn))
+    got[np.repeat(np.arange(R), np.diff(rp)), ci] = val
+    assert np.all(np.diff(rp) >= 0) and rp[-1] == len(ci)
+    for r in range(R):
+        assert np.all(np.diff(ci[rp[r]:rp[r + 1]]) > 0)  # columns ascending, merged
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+    # no levels: the block itself
+    rp0, ci0, val0 = off.csr_fold_levels(to_csr(dense), [])
+    base = to_csr(dense)
+    assert np.array_equal(rp0, base[0]) and np.array_equal(ci0, base[1]) and np.array_equal(val0, base[2])
+    # a level that reads a row it writes is refused
+    bad = np.zeros((R, R), np.float32)
+    bad[5, 6] = bad[6, 7] = 1
+    with pytest.raises(RuntimeError):
+        off.csr_fold_levels(to_csr(dense), [to_csr(bad)])
