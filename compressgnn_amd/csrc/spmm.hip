@@ -49,7 +49,7 @@ namespace {
 
 constexpr int kUnroll = 4;        // gathers in flight per lane and tile, nnz schedule (with 7 waves per SIMD;
                                   // 8 in flight with 5 waves measured the same)
-constexpr int kRowUnroll = 8;     // same for the row schedule (4: 9 % slower on web-graph out-lists, 12: 30 %)
+constexpr int kRowUnroll = 4;     // same for the row schedule (8: 9 % slower on web-graph out-lists, 2: 13 %, 16: 38 %)
 constexpr int kXcds = 8;          // accelerator dies of an MI355X, each with its own L2
 constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
 
