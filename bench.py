@@ -480,6 +480,21 @@ def main():
                                              forward_GBps=pb_f["bytes"] / (f_ms * 1e-3) / 1e9,
                                              backward_GBps=pb_b["bytes"] / (b_ms * 1e-3) / 1e9,
                                              forward_bytes=pb_f["bytes"], backward_bytes=pb_b["bytes"])
+    # the same kernels on a graph whose gathers stay in L2: row lengths and weights of the C1 graph,
+    # neighbours drawn from a window of 2,048 vertices around the row instead of the copy model
+    rng_l = np.random.default_rng(11)
+    src_l = np.repeat(np.arange(C1_VERTICES, dtype=np.int64), np.diff(v2))
+    col_l = (src_l + rng_l.integers(-1024, 1024, size=len(src_l))) % C1_VERTICES
+    col_l = col_l[np.argsort(src_l * C1_VERTICES + col_l, kind="stable")]
+    local = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(col_l), torch.from_numpy(w), C1_VERTICES,
+                         C1_VERTICES, dev)
+    lb = block_bytes(v2, col_l, C1_VERTICES, F, 0)
+    detail["windowed_graph_same_row_lengths"] = {}
+    for name in ("rowbalance", "nnzbalance"):
+        l_ms = time_loop(lambda: local.spmm(x, None, name), args.steps, 2, torch)
+        detail["windowed_graph_same_row_lengths"][name] = dict(ms=l_ms, bytes=lb["bytes"],
+                                                               GBps=lb["bytes"] / (l_ms * 1e-3) / 1e9)
+    del local
     # parity of the measured configuration: compressed == plain within tolerance
     out, gx = step()
     ref_out = plain_t.spmm(x, None, "rowbalance")

@@ -85,6 +85,8 @@ struct SpmmArgs {
     // Runs per workgroup of the nnz kernel that wrote carry_row/carry (its carries are
     // merged per workgroup: see kMerged), or 1 for the plain list a reduction level writes.
     int32_t merge_stride;
+    int32_t stretch_log2;  // log2 of the workgroups per XCD stretch (see logical_block); set at launch
+    int32_t blocks;        // workgroups with work (the grid rounds this up to a multiple of kXcds)
 };
 
 // carry_row values below zero: the run carries nothing, or its carry was added to that
@@ -236,27 +238,48 @@ __device__ __forceinline__ int out_row(const SpmmArgs<T> &a, int r) {
     return a.rowmap != nullptr ? a.rowmap[r] : r;
 }
 
-// Workgroups are dealt to the XCDs round robin.  With a locality order, XCD x takes every
-// kXcds-th stretch of consecutive workgroups' worth of stored rows (or runs): neighbours in
-// the order meet in one L2, and every XCD gets the same mix of the matrix (one contiguous
-// share each would leave the XCD with the least reuse to finish last).  A stretch holds
-// kXcdStretchGroups lane groups, about what an XCD holds at a time at F = 128, so an XCD works
-// on one region of the order at once (a quarter and twice that measured 1.5 % slower on the
-// web graph, four times 20 %: too few stretches to even out).  The grid is a multiple of
-// kXcds stretches.
+// Workgroups are dealt to the XCDs round robin.  XCD x takes every kXcds-th stretch of
+// consecutive workgroups' worth of stored rows (or runs): rows that follow each other in the
+// store (a locality order, or a natural order that has locality) meet in one L2, and every
+// XCD gets the same mix of the matrix (one contiguous share each would leave the XCD with the
+// least reuse to finish last).  A stretch holds kXcdStretchGroups lane groups, about what an
+// XCD holds at a time at F = 128, so an XCD works on one region of the order at once (a
+// quarter and twice that measured 1.5 % slower on the web graph, four times 20 %: too few
+// stretches to even out).  Small launches take shorter stretches, at least
+// kMinStretchesPerXcd per XCD.
 constexpr int kXcdStretchGroups = 2048;
+constexpr int kMinStretchesPerXcd = 6;
 
 template <int GPB>
 constexpr int xcd_stretch() {
     return kXcdStretchGroups / GPB > 0 ? kXcdStretchGroups / GPB : 1;
 }
 
-template <int GPB, typename T>
+// log2 of the stretch (in workgroups) for a launch of `blocks` workgroups of GPB lane groups
+template <int GPB>
+int stretch_log2_for(int64_t blocks) {
+    int lg = 0;
+    while ((2 << lg) <= xcd_stretch<GPB>()) ++lg;
+    while (lg > 0 && blocks < ((int64_t)kXcds * kMinStretchesPerXcd << lg)) --lg;
+    return lg;
+}
+
+// Whole rounds of kXcds stretches are dealt first; what is left over is dealt the same way in
+// stretches half as long, and so on down to single workgroups, so that no XCD is left with a
+// whole stretch more than another.
+template <typename T>
 __device__ __forceinline__ int logical_block(const SpmmArgs<T> &a) {
-    if (a.rowmap == nullptr) return blockIdx.x;
-    constexpr int kStretch = xcd_stretch<GPB>();
-    const int xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;  // turn: this workgroup's number on its XCD
-    return ((turn / kStretch) * kXcds + xcd) * kStretch + turn % kStretch;
+    const int xcd = blockIdx.x % kXcds;
+    int turn = blockIdx.x / kXcds;  // this workgroup's number on its XCD
+    int base = 0, left = a.blocks;
+    for (int lg = a.stretch_log2; lg > 0; --lg) {
+        const int share = (left >> (lg + 3)) << lg;  // workgroups per XCD dealt in stretches of 2^lg  (kXcds = 2^3)
+        if (turn < share) return base + ((((turn >> lg) * kXcds) + xcd) << lg) + (turn & ((1 << lg) - 1));
+        turn -= share;
+        base += share * kXcds;
+        left -= share * kXcds;
+    }
+    return base + turn * kXcds + xcd;
 }
 
 // ---------------------------------------------------------------- row schedule --
@@ -264,7 +287,7 @@ template <typename T, int VEC, int LPR, int TILES, int MODE>
 __global__ __launch_bounds__(kBlock) void spmm_row_kernel(SpmmArgs<T> a) {
     constexpr int GPB = kBlock / LPR;
     const int lane = threadIdx.x % LPR;
-    int row = logical_block<GPB>(a) * GPB + threadIdx.x / LPR;
+    int row = logical_block(a) * GPB + threadIdx.x / LPR;
     if constexpr (LPR == kWave) row = __builtin_amdgcn_readfirstlane(row);
     if (row >= a.rows) return;
     const int e0 = a.rowptr[row], e1 = a.rowptr[row + 1];
@@ -373,7 +396,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     __shared__ int wg_row[GPB];
     __shared__ Pack<T, VEC> wg_carry[TILES][kBlock];
     const int lane = threadIdx.x % LPR, grp = threadIdx.x / LPR;
-    int seg = logical_block<GPB>(a) * GPB + grp;
+    int seg = logical_block(a) * GPB + grp;
     if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
     int e0 = 0, e1 = 0;
     if (seg < a.nseg) {
@@ -796,12 +819,17 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
 enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2, KIND_REDUCE = 3 };
 
 template <typename T, int VEC, int LPR, int TILES>
-int launch_shape(int kind, int mode, const SpmmArgs<T> &a, int64_t items, int grid_y, hipStream_t stream) {
+int launch_shape(int kind, int mode, const SpmmArgs<T> &args, int64_t items, int grid_y, hipStream_t stream) {
     constexpr int GPB = kBlock / LPR;
     dim3 grid((unsigned)ceil_div(items, GPB), (unsigned)grid_y), block(kBlock);
     if (grid.x == 0) return CGNN_OK;
-    if ((kind == KIND_ROW || kind == KIND_NNZ) && a.rowmap != nullptr)
-        grid.x = (unsigned)(ceil_div(grid.x, kXcds * xcd_stretch<GPB>()) * kXcds * xcd_stretch<GPB>());
+    SpmmArgs<T> a = args;
+    a.stretch_log2 = 0;
+    if (kind == KIND_ROW || kind == KIND_NNZ) {
+        a.stretch_log2 = stretch_log2_for<GPB>(grid.x);
+        a.blocks = (int32_t)grid.x;
+        grid.x = (unsigned)(ceil_div((int64_t)grid.x, kXcds) * kXcds);
+    }
     switch (kind) {
         case KIND_ROW:
             if (mode == MODE_DUAL)
