@@ -25,7 +25,7 @@ EXPORTS = [
     "cgnn_lsh_group_workspace_bytes", "cgnn_lsh_group",
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
     "cgnn_cluster_mean_workspace_bytes", "cgnn_cluster_mean", "cgnn_cluster_mean_backward",
-    "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_copy_bytes", "cgnn_read_bytes",
+    "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_copy_bytes", "cgnn_read_bytes", "cgnn_fill_bytes",
 ]
 
 

@@ -882,6 +882,14 @@ __global__ __launch_bounds__(kBlock) void read16_kernel(const probe_word_t *__re
     if (acc == 0x9e3779b9u) *sink = acc;  // keeps the loads alive; practically never taken
 }
 
+// Writes n 16-byte words of zeros with streaming stores: the memory system's write rate.
+__global__ __launch_bounds__(kBlock) void fill16_kernel(probe_word_t *__restrict__ dst, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const probe_word_t zero = {0u, 0u, 0u, 0u};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        __builtin_nontemporal_store(zero, dst + i);
+}
+
 int check_bits(int bits) {
     if (bits < 0 || bits > 30) return fail(CGNN_EINVAL, "hash bits must be in [0,30]");
     return CGNN_OK;
@@ -1087,6 +1095,17 @@ extern "C" int cgnn_read_bytes(const void *src, size_t n, void *sink, cgnn_strea
     hipLaunchKernelGGL(read16_kernel, dim3(2u * (unsigned)compute_units()), dim3(kBlock), 0, stream,
                        static_cast<const probe_word_t *>(src), n / 16, static_cast<uint32_t *>(sink));
     return check_launch("read_bytes");
+}
+
+extern "C" int cgnn_fill_bytes(void *dst, size_t n, cgnn_stream_t stream) {
+    CGNN_REQUIRE(n % 16 == 0, "cgnn_fill_bytes: size must be a multiple of 16");
+    if (n == 0) return CGNN_OK;
+    CGNN_REQUIRE(dst, "cgnn_fill_bytes: null pointer");
+    size_t blocks = (n / 16 + kBlock - 1) / kBlock;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(fill16_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                       static_cast<probe_word_t *>(dst), n / 16);
+    return check_launch("fill_bytes");
 }
 
 extern "C" int cgnn_copy_bytes(const void *src, void *dst, size_t n, cgnn_stream_t stream) {

@@ -237,6 +237,11 @@ int cgnn_copy_bytes(const void *src, void *dst, size_t n, cgnn_stream_t stream);
  * which is what the gather-bound kernels are compared with. */
 int cgnn_read_bytes(const void *src, size_t n, void *sink, cgnn_stream_t stream);
 
+/* A plain streaming write of n bytes of zeros (n % 16 == 0): the write rate the memory
+ * system sustains, which is what the write-bound kernels (reconstruct, the gradient of the
+ * means) are compared with. */
+int cgnn_fill_bytes(void *dst, size_t n, cgnn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -205,3 +205,22 @@ def test_large_cluster_sums():
     rg = abi.reconstruct_backward(_t(go), _t(out), members, 9, True).cpu().numpy()
     want = oracle.reconstruct_backward(go.astype(np.float64), ids_np, out.astype(np.float64), 9, True)
     np.testing.assert_allclose(rg, want, rtol=1e-4, atol=1e-3)
+
+
+def test_memory_probes_move_what_they_say():
+    """The calibration kernels: the copy reproduces its source, the fill writes zeros over exactly n bytes."""
+    import ctypes
+    L = abi.lib()
+    n = 16 * 100003
+    src = torch.randint(1, 255, (n + 16,), dtype=torch.uint8, device=DEV)
+    dst = torch.full((n + 16,), 7, dtype=torch.uint8, device=DEV)
+    abi.check(L.cgnn_copy_bytes(abi.ptr(src), abi.ptr(dst), ctypes.c_size_t(n), abi.stream_of(src)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n], src[:n]) and bool((dst[n:] == 7).all())
+    abi.check(L.cgnn_fill_bytes(abi.ptr(dst), ctypes.c_size_t(n), abi.stream_of(dst)))
+    torch.cuda.synchronize()
+    assert int(dst[:n].count_nonzero()) == 0 and bool((dst[n:] == 7).all())
+    sink = torch.zeros(1, dtype=torch.int32, device=DEV)
+    abi.check(L.cgnn_read_bytes(abi.ptr(src), ctypes.c_size_t(n), abi.ptr(sink), abi.stream_of(src)))
+    torch.cuda.synchronize()
+    assert L.cgnn_fill_bytes(abi.ptr(dst), ctypes.c_size_t(7), abi.stream_of(dst)) != 0
