@@ -87,6 +87,7 @@ struct SpmmArgs {
     int32_t merge_stride;
     int32_t stretch_log2;  // log2 of the workgroups per XCD stretch (see logical_block); set at launch
     int32_t blocks;        // workgroups with work (the grid rounds this up to a multiple of kXcds)
+    int32_t read_once;     // MODE_UNIT: every row of X is gathered once (member lists), so with streaming loads
 };
 
 // carry_row values below zero: the run carries nothing, or its carry was added to that
@@ -97,6 +98,20 @@ constexpr int kMerged = -2;
 template <typename T, int VEC>
 __device__ __forceinline__ Pack<T, VEC> load_pack(const T *p) {
     return *reinterpret_cast<const Pack<T, VEC> *>(p);
+}
+// Streaming load for rows that this launch reads once.
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> load_pack_stream(const T *p) {
+    Pack<T, VEC> x;
+    if constexpr (VEC == 1) {
+        x.v[0] = __builtin_nontemporal_load(p);
+    } else {
+        typedef T vec_t __attribute__((ext_vector_type(VEC)));
+        const vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p));
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = v[i];
+    }
+    return x;
 }
 template <typename T, int VEC>
 __device__ __forceinline__ void store_pack(T *p, const Pack<T, VEC> &x) {
@@ -223,9 +238,11 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
         }
     }
     const int64_t off = (int64_t)c * (int32_t)a.F + foff;  // F < 2^31: one 32 x 32 -> 64 bit multiply
-    x = load_pack<T, VEC>(base + off);
+    // rows that are gathered once (member lists; masks exist for those only) are not kept in the caches
+    if (MODE == MODE_RELU_MASK || (MODE == MODE_UNIT && a.read_once)) x = load_pack_stream<T, VEC>(base + off);
+    else x = load_pack<T, VEC>(base + off);
     if constexpr (MODE == MODE_RELU_MASK) {
-        Pack<T, VEC> m = load_pack<T, VEC>(a.M + off);
+        Pack<T, VEC> m = load_pack_stream<T, VEC>(a.M + off);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) x.v[i] = (m.v[i] <= T(0)) ? T(0) : x.v[i];
     }
@@ -989,6 +1006,7 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     if (A->rows == 0 || F == 0) return CGNN_OK;
     if (mode != MODE_DUAL) split = INT32_MAX;  // every column comes from X
     SpmmArgs<T> a = make_args<T>(A, X, X1, split, M, Y, F, accumulate);
+    a.read_once = mode == MODE_UNIT || mode == MODE_RELU_MASK;  // asked for by name: the cluster reductions
     kernel = resolve_kernel(A, kernel);
     if (mode == MODE_RELU_MASK) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
     if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;
