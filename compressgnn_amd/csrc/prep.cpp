@@ -14,6 +14,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <deque>
 #include <numeric>
 #include <parallel/algorithm>
 #include <stdexcept>
@@ -232,54 +233,89 @@ cgnn_arrays *topo_partition(i64 R, const i64 *vlist, const i64 *elist, const flo
 
 // ------------------------------------------------------------------ rule filters --
 
-Rows rows_of(i64 n, const i64 *vlist, const i64 *elist) {
-    Rows g(n);
-    for (i64 v = 0; v < n; ++v) g[v].assign(elist + vlist[v], elist + vlist[v + 1]);
-    return g;
-}
+// The rows of the compressed graph while rules are being inlined.  A row lives in the
+// input arrays until it changes; only the rows that refer to an inlined rule (and the
+// rules themselves) are ever copied out, so a filter pass costs a scan of the input plus
+// work in proportion to what it inlines.
+class EditedRows {
+  public:
+    EditedRows(i64 n, const i64 *vlist, const i64 *elist) : vlist_(vlist), elist_(elist), slot_(n, -1) {}
+    i64 size_of(i64 n) const { return slot_[n] < 0 ? vlist_[n + 1] - vlist_[n] : (i64)edited_[slot_[n]].size(); }
+    std::vector<i64> &edit(i64 n) {
+        if (slot_[n] < 0) {
+            slot_[n] = (int32_t)edited_.size();
+            edited_.emplace_back(elist_ + vlist_[n], elist_ + vlist_[n + 1]);
+        }
+        return edited_[slot_[n]];
+    }
+    template <typename F>
+    void for_each(i64 n, F f) const {
+        if (slot_[n] < 0)
+            for (i64 e = vlist_[n]; e < vlist_[n + 1]; ++e) f(elist_[e]);
+        else
+            for (i64 c : edited_[slot_[n]]) f(c);
+    }
 
-Rows referrers_of(i64 n, const i64 *vlist, const i64 *elist) {
-    Rows t(n);
-    for (i64 v = 0; v < n; ++v)
-        for (i64 e = vlist[v]; e < vlist[v + 1]; ++e) t[elist[e]].push_back(v);
+  private:
+    const i64 *vlist_, *elist_;
+    std::vector<int32_t> slot_;
+    std::deque<std::vector<i64>> edited_;  // a deque: rows handed out by edit() stay where they are
+};
+
+// For every rule, the rows that refer to it, in ascending row order (one entry per
+// reference).  The referrers of vertices are not kept: no filter decision reads them.
+Rows rule_referrers(i64 V, i64 R, const i64 *vlist, const i64 *elist) {
+    Rows t(R);
+    for (i64 v = 0; v < V + R; ++v)
+        for (i64 e = vlist[v]; e < vlist[v + 1]; ++e)
+            if (elist[e] >= V) t[elist[e] - V].push_back(v);
     return t;
 }
 
 // Splice rule `id` into every row that refers to it (children keep their order and
-// take the place of the reference), and let its children refer to those rows instead.
+// take the place of the reference), and let its rule children refer to those rows instead.
 // Reference: src/offline/csrc/filter.h:30-66 / depth_filter.h:16-38.  `on_parent` and
 // `on_child` see the rows whose statistics the caller tracks.
 template <typename FP, typename FC>
-void inline_rule(i64 id, Rows &g, Rows &gt, FP on_parent, FC on_child) {
-    for (size_t i = 0; i < gt[id].size(); ++i) {
-        const i64 parent = gt[id][i];
-        auto it = std::find(g[parent].begin(), g[parent].end(), id);
-        auto pos = g[parent].erase(it);
-        g[parent].insert(pos, g[id].begin(), g[id].end());
+void inline_rule(i64 id, i64 V, EditedRows &g, Rows &gt, FP on_parent, FC on_child) {
+    std::vector<i64> body;  // a copy: no reference into the container is held while rows are copied out
+    g.for_each(id, [&](i64 c) { body.push_back(c); });
+    const std::vector<i64> &referrers = gt[id - V];
+    for (size_t i = 0; i < referrers.size(); ++i) {
+        const i64 parent = referrers[i];
+        std::vector<i64> &row = g.edit(parent);
+        auto pos = row.erase(std::find(row.begin(), row.end(), id));
+        row.insert(pos, body.begin(), body.end());
         on_parent(parent);
     }
-    for (size_t i = 0; i < g[id].size(); ++i) {
-        const i64 child = g[id][i];
-        auto it = std::find(gt[child].begin(), gt[child].end(), id);
-        auto pos = gt[child].erase(it);
-        gt[child].insert(pos, gt[id].begin(), gt[id].end());
+    for (size_t i = 0; i < body.size(); ++i) {
+        const i64 child = body[i];
+        if (child < V) continue;
+        std::vector<i64> &refs = gt[child - V];
+        auto pos = refs.erase(std::find(refs.begin(), refs.end(), id));
+        refs.insert(pos, referrers.begin(), referrers.end());
         on_child(child);
     }
 }
 
 // Dense renumbering of the surviving rules and re-emission of all rows.
 // Reference: src/offline/csrc/util.h:108-119,143-164.
-cgnn_arrays *emit_filtered(const Rows &g, const std::vector<char> &dropped, i64 V, i64 R) {
+cgnn_arrays *emit_filtered(const EditedRows &g, const std::vector<char> &dropped, i64 V, i64 R) {
     std::vector<i64> new_id(R);
     i64 next = V;
     for (i64 r = 0; r < R; ++r) {
         new_id[r] = next;
         if (!dropped[r]) ++next;
     }
+    i64 total = 0;
+    for (i64 n = 0; n < V + R; ++n)
+        if (n < V || !dropped[n - V]) total += g.size_of(n);
     std::vector<i64> nv{0}, ne;
+    nv.reserve(next + 1);
+    ne.reserve(total);
     for (i64 n = 0; n < V + R; ++n) {
         if (n >= V && dropped[n - V]) continue;
-        for (i64 c : g[n]) ne.push_back(c >= V ? new_id[c - V] : c);
+        g.for_each(n, [&](i64 c) { ne.push_back(c >= V ? new_id[c - V] : c); });
         nv.push_back((i64)ne.size());
     }
     auto *out = new cgnn_arrays;
@@ -292,21 +328,22 @@ cgnn_arrays *emit_filtered(const Rows &g, const std::vector<char> &dropped, i64 
 
 // Reference: src/offline/csrc/filter.h:26-28,68-118.
 cgnn_arrays *filter_csr(i64 V, i64 R, const i64 *vlist, const i64 *elist, int threshold) {
-    Rows g = rows_of(V + R, vlist, elist), gt = referrers_of(V + R, vlist, elist);
+    EditedRows g(V + R, vlist, elist);
+    Rows gt = rule_referrers(V, R, vlist, elist);
     std::vector<int> len(R), freq(R);
     std::vector<char> drop(R);
     auto small_saving = [&](int l, int f) { return (f - 1) * (l - 1) - 1 <= threshold; };
     for (i64 r = 0; r < R; ++r) {
-        freq[r] = (int)gt[r + V].size();
-        len[r] = (int)g[r + V].size();
+        freq[r] = (int)gt[r].size();
+        len[r] = (int)g.size_of(r + V);
         drop[r] = small_saving(len[r], freq[r]);
     }
     for (i64 r = 0; r < R; ++r) {
         if (!drop[r]) continue;
         const i64 id = r + V;
-        const int grow = (int)g[id].size() - 1;
+        const int grow = (int)g.size_of(id) - 1;
         inline_rule(
-            id, g, gt,
+            id, V, g, gt,
             [&](i64 parent) {
                 if (parent >= V) {
                     len[parent - V] += grow;
@@ -314,11 +351,9 @@ cgnn_arrays *filter_csr(i64 V, i64 R, const i64 *vlist, const i64 *elist, int th
                 }
             },
             [&](i64 child) {
-                if (child >= V) {
-                    // the reference adds the whole new referrer count here (filter.h:59)
-                    freq[child - V] += (int)gt[child].size();
-                    drop[child - V] = small_saving(len[child - V], freq[child - V]);
-                }
+                // the reference adds the whole new referrer count here (filter.h:59)
+                freq[child - V] += (int)gt[child - V].size();
+                drop[child - V] = small_saving(len[child - V], freq[child - V]);
             });
     }
     return emit_filtered(g, drop, V, R);
@@ -393,7 +428,8 @@ int vertex_order_csc(i64 V, i64 R, const i64 *vlist, const i64 *elist, std::vect
 
 // Reference: src/offline/csrc/depth_filter.h:40-116.
 cgnn_arrays *depth_filter_csr(i64 V, i64 R, const i64 *vlist, const i64 *elist, int max_depth, int min_edge) {
-    Rows g = rows_of(V + R, vlist, elist), gt = referrers_of(V + R, vlist, elist);
+    EditedRows g(V + R, vlist, elist);
+    Rows gt = rule_referrers(V, R, vlist, elist);
     std::vector<int32_t> depth;
     int deepest = vertex_order_csr(V, R, vlist, elist, depth);
     std::vector<char> drop(R, 0);
@@ -401,7 +437,7 @@ cgnn_arrays *depth_filter_csr(i64 V, i64 R, const i64 *vlist, const i64 *elist, 
     auto recount = [&](int upto) {
         for (int d = 0; d <= upto; ++d) edges_at[d] = 0;
         for (i64 r = 0; r < R; ++r)
-            if (!drop[r] && depth[r + V] <= deepest) edges_at[depth[r + V]] += (i64)g[r + V].size();
+            if (!drop[r] && depth[r + V] <= deepest) edges_at[depth[r + V]] += g.size_of(r + V);
     };
     for (i64 r = 0; r < R; ++r)
         if (depth[r + V] > deepest) {
@@ -417,7 +453,7 @@ cgnn_arrays *depth_filter_csr(i64 V, i64 R, const i64 *vlist, const i64 *elist, 
         }
         for (i64 r = 0; r < R; ++r)
             if (depth[r + V] == d) {
-                inline_rule(r + V, g, gt, [](i64) {}, [](i64) {});
+                inline_rule(r + V, V, g, gt, [](i64) {}, [](i64) {});
                 drop[r] = 1;
             }
         --d;
