@@ -803,8 +803,12 @@ int env_int(const char *name) {
 // alignment allow, then as many lanes as a row needs (power of two, 4..64).
 // CGNN_SPMM_VEC / CGNN_SPMM_LPR (environment, read once) override the choice where the
 // result is a layout that exists; they are for tuning experiments.
+// min_lpr: narrow the vectors (down to single words) while a row would take fewer lanes than
+// this.  The nnz schedule asks for 16: with 4 lanes per run a wave walks 16 runs at once, each
+// with its own row changes (F = 16: 0.106 -> 0.089 ms for the forward vertex stage of the web
+// graph); the row schedule is faster with the widest vectors (0.036 against 0.053 ms).
 template <typename T>
-Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, const void *p3) {
+Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, const void *p3, int min_lpr = 4) {
     static const int force_vec = env_int("CGNN_SPMM_VEC"), force_lpr = env_int("CGNN_SPMM_LPR");
     auto aligned = [&](size_t bytes) {
         auto ok = [&](const void *p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0; };
@@ -815,6 +819,7 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
     if (sizeof(T) == 4) {
         if (F % 4 == 0 && aligned(16)) s.vec = 4;
         else if (F % 2 == 0 && aligned(8)) s.vec = 2;
+        while (s.vec > 1 && F / s.vec < min_lpr) s.vec /= 2;
         if (force_vec == 2 && s.vec == 4) s.vec = 2;
         if (force_vec == 1) s.vec = 1;
     }
@@ -1021,7 +1026,7 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     const int64_t nseg = ceil_div(A->nnz, seg);
     // the lane layout decides how many runs a workgroup merges (the carries sit at multiples
     // of 256 bytes in the workspace, so the workspace stands for them in the alignment check)
-    const Shape s = pick_shape<T>(F, X, Y, ws, mode == MODE_DUAL ? X1 : M);
+    const Shape s = pick_shape<T>(F, X, Y, ws, mode == MODE_DUAL ? X1 : M, 16);
     const int runs_per_workgroup = kBlock / s.lpr;
     const CarryLevels levels = carry_levels(nseg, F, sizeof(T), wants_levels(A, seg, runs_per_workgroup));
     if (nseg > 0 && (ws == nullptr || ws_bytes < levels.total)) {
