@@ -28,7 +28,7 @@ def _run(vlist, elist, value, x, kernel, out0=None, seg=0):
     return Y.cpu().numpy()
 
 
-@pytest.mark.parametrize("F", [1, 3, 4, 16, 31, 33, 64, 100, 128, 130, 256, 512, 602])
+@pytest.mark.parametrize("F", [1, 3, 4, 8, 16, 31, 32, 33, 64, 100, 128, 130, 256, 512, 602])
 @pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
 def test_spmm_matches_oracle(F, kernel):
     rng = np.random.default_rng(100 + F)
@@ -43,6 +43,23 @@ def test_spmm_matches_oracle(F, kernel):
     want2 = oracle.spmm(vlist, elist, value, x, out0.copy())
     got2 = _run(vlist, elist, value, x, kernel, out0)
     assert np.array_equal(got2, want2)
+
+
+@pytest.mark.parametrize("rows", [2047, 20011, 70001])
+@pytest.mark.parametrize("F", [16, 128])
+@pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
+def test_launches_of_many_workgroups(rows, F, kernel):
+    """Grids of tens to thousands of workgroups: the workgroups are renumbered before they
+    pick their rows (stretches of the store per XCD, leftovers in shorter stretches), and
+    every row must still be computed exactly once.  Rows are short, so the result is
+    bit-identical to the sequential sum under both schedules."""
+    rng = np.random.default_rng(rows + F)
+    vlist, elist, value = random_csr(rng, rows, 3000, 3.0)
+    x = rng.standard_normal((3000, F)).astype(np.float32)
+    want = oracle.spmm(vlist, elist, value, x)
+    assert np.array_equal(_run(vlist, elist, value, x, kernel), want)
+    out0 = rng.standard_normal((rows, F)).astype(np.float32)
+    assert np.array_equal(_run(vlist, elist, value, x, kernel, out0), oracle.spmm(vlist, elist, value, x, out0.copy()))
 
 
 @pytest.mark.parametrize("seg", [8, 64, 256])
