@@ -1,8 +1,12 @@
-"""Reconstruct node features from representatives, optionally fusing the shared bias
-and ReLU (reference layer/CompressgnnReconstruct.py:11-42).  The gradient with respect
-to the representatives is a per-cluster sum; it runs on the member lists recorded by
-Compressgnn_Cluster for the index tensor when they are available, and builds them on the
-fly otherwise."""
+"""Node features from cluster representatives: out[i] = act(src[index[i]] + bias).
+
+Module Compressgnn_Reconstruct with the call signature of the reference's
+layer/CompressgnnReconstruct.py:29-42.  On the GPU the gather, the bias and the ReLU are
+one kernel; the gradient for the representatives is a per-cluster sum of the (masked)
+output gradient, taken over the member lists that Compressgnn_Cluster recorded for the
+index tensor, or over lists built on the spot for an index from elsewhere.  The bias
+gradient is the column sum of that (layer/CompressgnnReconstruct.py:26).
+"""
 import _paths  # noqa: F401
 import torch
 from torch.autograd.function import once_differentiable
@@ -10,25 +14,33 @@ from torch.autograd.function import once_differentiable
 import compressgnn_runtime as _native
 from CompressgnnCluster import members_of
 
+_ACTIVATIONS = (None, 'relu')
 
-class _Reconstruct(torch.autograd.Function):
+
+def _dense(t):
+    return None if t is None else t.contiguous()
+
+
+class _GatherBiasAct(torch.autograd.Function):
+    """(representatives[C, F], ids[N], bias[F] or None, relu) -> rows[N, F]"""
+
     @staticmethod
-    def forward(ctx, src, index, bias, relu):
-        index = index.contiguous()
-        ctx.members = members_of(index, src.size(0))
-        output = _native.cluster_reconstruct(src.contiguous(), index, None if bias is None else bias.contiguous(),
-                                             relu, ctx.members)
-        ctx.save_for_backward(index, output)
-        ctx.groups, ctx.relu, ctx.has_bias = src.size(0), relu, bias is not None
-        return output
+    def forward(ctx, reps, ids, bias, relu):
+        ids = _dense(ids)
+        lists = members_of(ids, reps.size(0))
+        rows = _native.cluster_reconstruct(_dense(reps), ids, _dense(bias), relu, lists)
+        # the ReLU mask of the gradient is read off the rows that were produced
+        ctx.save_for_backward(ids, rows)
+        ctx.plan = (reps.size(0), relu, bias is not None, lists)
+        return rows
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, grad):
-        index, output = ctx.saved_tensors
-        reps_grad = _native.cluster_reconstruct_backward(grad.contiguous(), index, output, ctx.groups, ctx.relu,
-                                                         ctx.members)
-        return reps_grad, None, reps_grad.sum(0) if ctx.has_bias else None, None
+    def backward(ctx, d_rows):
+        clusters, relu, with_bias, lists = ctx.plan
+        ids, rows = ctx.saved_tensors
+        d_reps = _native.cluster_reconstruct_backward(_dense(d_rows), ids, rows, clusters, relu, lists)
+        return d_reps, None, (d_reps.sum(0) if with_bias else None), None
 
 
 class Compressgnn_Reconstruct(torch.nn.Module):
@@ -36,15 +48,19 @@ class Compressgnn_Reconstruct(torch.nn.Module):
         super().__init__()
         self.node_dim = node_dim
 
+    def _kernel_applies(self, src):
+        # rows along the first axis of a matrix that lives on the GPU
+        return src.is_cuda and src.dim() == 2 and self.node_dim in (0, -2)
+
     def forward(self, src, index, bias=None, activation=None):
-        if activation not in (None, 'relu'):
-            raise ValueError('Supported activations: None, relu')
-        if src.is_cuda and src.dim() == 2 and self.node_dim in (0, -2):
-            # the reference takes its fused kernel only when there is a bias or an
-            # activation to fuse (layer/CompressgnnReconstruct.py:37); the plain gather
-            # is the same kernel here
-            return _Reconstruct.apply(src, index, bias, activation == 'relu')
-        output = src.index_select(self.node_dim, index)
-        if bias is not None:
-            output = output + bias
-        return output.relu() if activation == 'relu' else output
+        if activation not in _ACTIVATIONS:
+            raise ValueError("activation must be None or 'relu'")
+        relu = activation is not None
+        if self._kernel_applies(src):
+            # one kernel with or without bias / activation (the reference switches to its
+            # fused kernel only when there is something to fuse, :37)
+            return _GatherBiasAct.apply(src, index, bias, relu)
+        # anything else (other layouts, host tensors) is plain tensor algebra
+        rows = src.index_select(self.node_dim, index)
+        rows = rows if bias is None else rows + bias
+        return rows.relu() if relu else rows

@@ -1,39 +1,49 @@
-"""CompressgnnData: builds the compressed, normalised, partitioned graph from raw
-arrays.  Same constructor, fields, to() and __repr__ as the reference's
-loader/CompressgnnData.py:60-201: graph_type="csr" yields a CompressGraph, graph_type="coo"
-per-phase edge lists and weights."""
+"""CompressgnnData: from raw arrays to the compressed, normalised, partitioned graph.
+
+The constructor arguments, the fields it leaves on the object (x, y, the three masks,
+vertex_cnt, rule_cnt, edge_cnt, feature_dim, graph_type, step, edge_index, edge_weight for
+"coo", and the compression settings), to() and the text of __repr__ are those of the
+reference's loader/CompressgnnData.py:60-201.  graph_type="csr" ends in a CompressGraph,
+graph_type="coo" in one [2, E_k] edge tensor and one weight vector per phase.
+
+Pipeline (the reference's order): self loops -> normalised degrees of the uncompressed
+graph -> batch compression -> saving filter -> depth filter -> weights of the compressed
+edges -> partition ("csr") or phase masks ("coo").
+"""
 import _paths  # noqa: F401
 import numpy as np
 import torch
 
-from compressgnn_offline import (add_self_loop_coo, add_self_loop_csr, coo2csr, csr2coo, csr_transpose,
-                                 depth_filter_csr, filter_csr, gcn_norm_coo_compress, gcn_norm_csr_compress,
-                                 gen_mask_edge, gen_vertex_order_csc, get_norm_degree)
+import compressgnn_offline as offline
 from compress_graph import CompressGraph
 from compression_backend import compress_graph_csr, resolve_backend
 
 
+def _size(vlist, elist):
+    return int(vlist.shape[0]) + int(elist.shape[0])
+
+
 def compress(vlist, elist, threshold, max_depth, min_edge, min_pair_frequency=16,
              compression_backend='auto', compression_threads=4, compression_rounds=12, verbose=True):
-    """Batch compression, then the saving filter, then the depth filter
-    (reference loader/CompressgnnData.py:26-55)."""
-    say = print if verbose else (lambda *a, **k: None)
-    selected = resolve_backend(compression_backend)
-    say('Compression backend: {}'.format(selected))
-    before = vlist.shape[0] + elist.shape[0]
-    result = compress_graph_csr(vlist, elist, min_pair_frequency, selected, compression_threads, compression_rounds)
-    new_vlist, new_elist, new_vertex_cnt, new_rule_cnt = result
-    say("compression ratio: {} / {} = {:.4f}".format(before, new_vlist.shape[0] + new_elist.shape[0],
-                                                     before / (new_vlist.shape[0] + new_elist.shape[0])))
-    new_vlist, new_elist, new_vertex_cnt, new_rule_cnt = filter_csr(
-        new_vlist, new_elist, new_vertex_cnt, new_rule_cnt, threshold)
-    say("After filter compression ratio: {} / {} = {:.4f}".format(
-        before, new_vlist.shape[0] + new_elist.shape[0], before / (new_vlist.shape[0] + new_elist.shape[0])))
-    new_vlist, new_elist, new_vertex_cnt, new_rule_cnt = depth_filter_csr(
-        new_vlist, new_elist, new_vertex_cnt, new_rule_cnt, max_depth, min_edge)
-    say("After depth filter compression ratio: {} / {} = {:.4f}".format(
-        before, new_vlist.shape[0] + new_elist.shape[0], before / (new_vlist.shape[0] + new_elist.shape[0])))
-    return new_vlist, new_elist, new_vertex_cnt, new_rule_cnt
+    """Batch compression, saving filter, depth filter (loader/CompressgnnData.py:26-55 of the
+    reference).  Returns (vlist, elist, vertex_cnt, rule_cnt) of the compressed graph; with
+    verbose, prints the size ratio after every stage."""
+    backend = resolve_backend(compression_backend)
+    original = _size(vlist, elist)
+    stages = (
+        ('batch compression (%s)' % backend,
+         lambda g: compress_graph_csr(vlist, elist, min_pair_frequency, backend, compression_threads,
+                                      compression_rounds)),
+        ('saving filter', lambda g: offline.filter_csr(g[0], g[1], g[2], g[3], threshold)),
+        ('depth filter', lambda g: offline.depth_filter_csr(g[0], g[1], g[2], g[3], max_depth, min_edge)),
+    )
+    graph = None
+    for name, run in stages:
+        graph = run(graph)
+        if verbose:
+            now = _size(graph[0], graph[1])
+            print('%-28s size %d -> %d, ratio %.4f, %d rules' % (name, original, now, original / now, graph[3]))
+    return graph
 
 
 class CompressgnnData():
@@ -50,92 +60,83 @@ class CompressgnnData():
                  compression_threads: int = 4,
                  compression_rounds: int = 12,
                  verbose: bool = False):
-        x = np.asarray(x).astype(np.float32)
-        self.x = torch.as_tensor(x)
+        if graph_type not in ("coo", "csr"):
+            raise ValueError('graph_type must be "coo" or "csr"')
+        self.x = torch.as_tensor(np.asarray(x).astype(np.float32))
         self.y = torch.as_tensor(np.array(y))
-        self.train_mask = torch.as_tensor(train_mask)
-        self.vaild_mask = torch.as_tensor(vaild_mask)
-        self.test_mask = torch.as_tensor(test_mask)
-        self.vertex_cnt = self.x.size()[0]
-        self.feature_dim = self.x.size()[1]
+        for name, mask in (("train_mask", train_mask), ("vaild_mask", vaild_mask), ("test_mask", test_mask)):
+            setattr(self, name, torch.as_tensor(mask))
+        self.vertex_cnt, self.feature_dim = self.x.size()[0], self.x.size()[1]
         self.graph_type = graph_type
         self.min_pair_frequency = min_pair_frequency
         self.compression_backend = resolve_backend(compression_backend)
         self.compression_threads = compression_threads
         self.compression_rounds = compression_rounds
-        if self.graph_type == "csr":
-            vlist = np.asarray(edge_index[0]).astype(np.int64)
-            elist = np.asarray(edge_index[1]).astype(np.int64)
-            if add_self_loop:
-                vlist, elist = add_self_loop_csr(vlist, elist)
-            if normalize:
-                norm_degree = get_norm_degree(elist, self.vertex_cnt)
-            new_vlist, new_elist, vertex_cnt, rule_cnt = compress(
-                vlist, elist, threshold, max_depth, min_edge, min_pair_frequency,
-                self.compression_backend, compression_threads, compression_rounds, verbose)
-            self.vertex_cnt = vertex_cnt
-            self.rule_cnt = rule_cnt
-            self.edge_cnt = new_elist.shape[0]
-            new_vlist = new_vlist.astype(np.int64)
-            new_elist = new_elist.astype(np.int64)
-            if normalize:
-                edge_weight = gcn_norm_csr_compress(new_vlist, new_elist, norm_degree, self.vertex_cnt, self.rule_cnt)
-            else:
-                edge_weight = np.ones(self.edge_cnt, dtype=np.float32)
-            # the phase count the reference reports (gen_mask_vertex(..., "csc"),
-            # loader/CompressgnnData.py:177-179); the kernels use CompressGraph.step instead
-            _, self.step = gen_vertex_order_csc(new_vlist, new_elist, self.vertex_cnt, self.rule_cnt)
-            total = vertex_cnt + rule_cnt
-            colptr, row, value = csr_transpose(new_vlist, new_elist, edge_weight, total)
-            self.edge_index = CompressGraph(colptr, row, value, self.vertex_cnt)
-        elif self.graph_type == "coo":
-            # reference loader/CompressgnnData.py:86-139: edges sorted by source
-            src = np.asarray(edge_index[0]).astype(np.int64)
-            dst = np.asarray(edge_index[1]).astype(np.int64)
-            if add_self_loop:
-                src, dst = add_self_loop_coo(src, dst, self.vertex_cnt)
-            if normalize:
-                norm_degree = get_norm_degree(dst, self.vertex_cnt)
-            vlist, elist = coo2csr(src, dst, self.vertex_cnt)
-            new_vlist, new_elist, new_vertex_cnt, new_rule_cnt = compress(
-                vlist, elist, threshold, max_depth, min_edge, min_pair_frequency,
-                self.compression_backend, compression_threads, compression_rounds, verbose)
-            self.vertex_cnt = new_vertex_cnt
-            self.rule_cnt = new_rule_cnt
-            self.edge_cnt = new_elist.shape[0]
-            src, dst = csr2coo(new_vlist, new_elist)
-            if normalize:
-                edge_weight = gcn_norm_coo_compress(src, dst, norm_degree, self.vertex_cnt, self.rule_cnt)
-            else:
-                edge_weight = np.ones(self.edge_cnt, dtype=np.float32)
-            edge_mask, step = gen_mask_edge(src, dst, self.vertex_cnt, self.rule_cnt)
-            if verbose:
-                print("step:{}".format(step))
-            self.step = step
-            pairs = torch.from_numpy(np.vstack((src, dst)))
-            weights = torch.from_numpy(edge_weight)
-            self.edge_index, self.edge_weight = [], []
-            for i in range(step):
-                mask = torch.from_numpy(edge_mask[i])
-                self.edge_index.append(torch.stack((pairs[0][mask], pairs[1][mask]), 0))
-                self.edge_weight.append(weights[mask])
+        self._settings = dict(threshold=threshold, max_depth=max_depth, min_edge=min_edge,
+                              min_pair_frequency=min_pair_frequency, compression_backend=self.compression_backend,
+                              compression_threads=compression_threads, compression_rounds=compression_rounds,
+                              verbose=verbose)
+        first = np.asarray(edge_index[0]).astype(np.int64)
+        second = np.asarray(edge_index[1]).astype(np.int64)
+        if graph_type == "csr":
+            self._from_csr(first, second, add_self_loop, normalize)
         else:
-            raise ValueError('graph_type must be "coo" or "csr"')
+            self._from_edges(first, second, add_self_loop, normalize, verbose)
+
+    def _compressed(self, vlist, elist):
+        vlist, elist, self.vertex_cnt, self.rule_cnt = compress(vlist, elist, **self._settings)
+        self.edge_cnt = elist.shape[0]
+        return vlist.astype(np.int64), elist.astype(np.int64)
+
+    # graph_type="csr": (vlist, elist) -> CompressGraph  (loader/CompressgnnData.py:140-181)
+    def _from_csr(self, vlist, elist, add_self_loop, normalize):
+        if add_self_loop:
+            vlist, elist = offline.add_self_loop_csr(vlist, elist)
+        degree = offline.get_norm_degree(elist, self.vertex_cnt) if normalize else None
+        vlist, elist = self._compressed(vlist, elist)
+        if normalize:
+            weight = offline.gcn_norm_csr_compress(vlist, elist, degree, self.vertex_cnt, self.rule_cnt)
+        else:
+            weight = np.ones(self.edge_cnt, dtype=np.float32)
+        # `step` is the phase count the reference reports for this form (its
+        # gen_mask_vertex(..., "csc"), :177-179); the kernels go by CompressGraph.step
+        self.step = offline.gen_vertex_order_csc(vlist, elist, self.vertex_cnt, self.rule_cnt)[1]
+        nodes = self.vertex_cnt + self.rule_cnt
+        colptr, row, value = offline.csr_transpose(vlist, elist, weight, nodes)
+        self.edge_index = CompressGraph(colptr, row, value, self.vertex_cnt)
+
+    # graph_type="coo": (src, dst) -> edge and weight tensors per phase  (:86-139)
+    def _from_edges(self, src, dst, add_self_loop, normalize, verbose):
+        if add_self_loop:
+            src, dst = offline.add_self_loop_coo(src, dst, self.vertex_cnt)
+        degree = offline.get_norm_degree(dst, self.vertex_cnt) if normalize else None
+        vlist, elist = self._compressed(*offline.coo2csr(src, dst, self.vertex_cnt))
+        src, dst = offline.csr2coo(vlist, elist)
+        if normalize:
+            weight = offline.gcn_norm_coo_compress(src, dst, degree, self.vertex_cnt, self.rule_cnt)
+        else:
+            weight = np.ones(self.edge_cnt, dtype=np.float32)
+        phase_masks, self.step = offline.gen_mask_edge(src, dst, self.vertex_cnt, self.rule_cnt)
+        if verbose:
+            print("phases: %d" % self.step)
+        edges = torch.from_numpy(np.vstack((src, dst)))
+        weights = torch.from_numpy(weight)
+        self.edge_index, self.edge_weight = [], []
+        for k in range(self.step):
+            keep = torch.from_numpy(phase_masks[k])
+            self.edge_index.append(edges[:, keep].contiguous())
+            self.edge_weight.append(weights[keep])
 
     def __repr__(self):
-        return 'CompressgnnData(vertex_cnt:"%s", rule_cnt:"%s", edge_cnt:"%s", step:"%s", graph_type:"%s")' % (
-            self.vertex_cnt, self.rule_cnt, self.edge_cnt, self.step, self.graph_type)
+        shown = (self.vertex_cnt, self.rule_cnt, self.edge_cnt, self.step, self.graph_type)
+        return 'CompressgnnData(vertex_cnt:"%s", rule_cnt:"%s", edge_cnt:"%s", step:"%s", graph_type:"%s")' % shown
 
     def to(self, device):
-        self.x = self.x.to(device)
-        self.y = self.y.to(device)
-        self.train_mask = self.train_mask.to(device)
-        self.vaild_mask = self.vaild_mask.to(device)
-        self.test_mask = self.test_mask.to(device)
-        if self.graph_type == "coo":
-            for i in range(self.step):
-                self.edge_index[i] = self.edge_index[i].to(device)
-                self.edge_weight[i] = self.edge_weight[i].to(device)
-        else:
+        for name in ("x", "y", "train_mask", "vaild_mask", "test_mask"):
+            setattr(self, name, getattr(self, name).to(device))
+        if self.graph_type == "csr":
             self.edge_index = self.edge_index.to(device)
+        else:
+            self.edge_index = [e.to(device) for e in self.edge_index]
+            self.edge_weight = [w.to(device) for w in self.edge_weight]
         return self
