@@ -40,6 +40,18 @@ class CompressGraph():
     def __repr__(self):
         return 'CompressGraph'
 
+    # torch.save(data) of a prepared dataset, as the reference's genData scripts do
+    # (genData/createCompressDataset.py:98): the blocks are saved, the device plan is not
+    # (it is rebuilt on first use after loading).
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        state['_plan'] = None
+        return state
+
+    def __setstate__(self, state):
+        self.__dict__.update(state)
+        self._plan = None
+
     def blocks(self):
         return [self.v2v_graph, self.v2r_graph, self.r2v_graph] + list(self.r2r_graph)
 

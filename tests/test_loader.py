@@ -159,3 +159,23 @@ def test_coo_phases_cover_the_compressed_graph():
     np.add.at(want, d2, (nd[s2] * nd[d2])[:, None] * x[s2])
     np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-5)
     assert "coo" in repr(data) and data.to("cpu") is data
+
+
+def test_a_prepared_dataset_survives_torch_save(tmp_path):
+    """The reference stores prepared datasets with torch.save(data) (genData/createCompressDataset.py:98).
+    The file written here is this test's own, so loading it with the unpickler is in order."""
+    import compressgnn_offline as off
+    v, e = off.gen_copy_model(2000, 9.0, 0.7, 3)
+    mask = np.ones(2000, dtype=bool)
+    data = CompressgnnData(np.ones((2000, 3), np.float32), (v, e), np.zeros(2000, np.int64), mask, mask, mask,
+                           graph_type="csr", min_pair_frequency=3, compression_backend="cpu")
+    data.edge_index._plan = lambda: None  # stands for a device plan: not part of the file
+    path = str(tmp_path / "data_csr.pt")
+    torch.save(data, path)
+    again = torch.load(path, weights_only=False)
+    assert repr(again) == repr(data) and again.edge_index._plan is None
+    for name in ("v2v_graph", "v2r_graph", "r2v_graph"):
+        for a, b in zip(getattr(data.edge_index, name).csr(), getattr(again.edge_index, name).csr()):
+            assert torch.equal(a, b)
+    assert again.edge_index.step == data.edge_index.step
+    assert torch.equal(again.edge_index.vertex_degree, data.edge_index.vertex_degree)
