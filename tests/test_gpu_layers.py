@@ -179,6 +179,43 @@ def test_propagate_schedules_agree(fuse, method):
         assert np.array_equal(out.cpu().numpy(), want)  # sequential sums in every stage
 
 
+def test_propagation_replays_from_a_captured_graph():
+    """Forward and gradient propagation make no host read, no memset and no allocation outside
+    torch's allocator, so a step can be captured in a graph; every replay, with eager work and
+    synchronisations in between and new values in the captured inputs, gives the bits of the eager step."""
+    data, _ = _make_data("copy", 64, True, 3, seed=4)
+    data.to(DEV)
+    plan = data.edge_index.plan()
+    V = data.vertex_cnt
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(9)
+    x = torch.randn(V, 64, device=DEV, generator=gen)
+    g = torch.randn(V, 64, device=DEV, generator=gen)
+
+    def step():
+        return plan.forward(x), plan.backward(g)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_graph, gx_graph = step()
+    for _ in range(3):
+        x.copy_(torch.randn(V, 64, device=DEV, generator=gen))
+        g.copy_(torch.randn(V, 64, device=DEV, generator=gen))
+        assert torch.isfinite((x * 2).sum()).item()  # eager work and a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        out_eager, gx_eager = step()
+        torch.cuda.synchronize()
+        assert torch.equal(out_graph, out_eager) and torch.equal(gx_graph, gx_eager)
+
+
 def test_spmm_func_int64_api():
     """The reference's raw operator on int64 CSR tensors, all accepted method strings."""
     import compressgnn_runtime as rt
