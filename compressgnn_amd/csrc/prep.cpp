@@ -996,24 +996,59 @@ cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const i
         }
         // the closest relative of every row
         std::vector<int32_t> best((size_t)rows, -1), shared((size_t)rows, 0);
+        // Counting how often every other row turns up: a row with few candidates counts them
+        // in a small hash table that stays in the core's cache; only rows with many use the
+        // counter per row of the matrix (random accesses into an array of the size of the graph
+        // were most of the time of this step).  Both give the same (most, lowest row) answer.
+        constexpr int32_t kSlots = 8192, kSmall = kSlots / 2;
 #pragma omp parallel
         {
             std::vector<int32_t> count((size_t)rows, 0), touched;
+            std::vector<int32_t> key((size_t)kSlots, -1), hits((size_t)kSlots, 0), used;
 #pragma omp for schedule(dynamic, 1024)
             for (i64 r = 0; r < rows; ++r) {
-                touched.clear();
+                i64 candidates = 0;
                 for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) {
-                    const i64 c = elist[e];
-                    if (cstart[c + 1] - cstart[c] > hub_rows) continue;
-                    for (i64 q = cstart[c]; q < cstart[c + 1]; ++q) {
-                        const int32_t o = crow[q];
-                        if (o != r && count[o]++ == 0) touched.push_back(o);
-                    }
+                    const i64 d = cstart[elist[e] + 1] - cstart[elist[e]];
+                    if (d <= hub_rows) candidates += d;
                 }
                 int32_t b = -1, most = 0;
-                for (int32_t o : touched) {
-                    if (count[o] > most || (count[o] == most && o < b)) most = count[o], b = o;
-                    count[o] = 0;
+                if (candidates <= kSmall) {
+                    used.clear();
+                    for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) {
+                        const i64 c = elist[e];
+                        if (cstart[c + 1] - cstart[c] > hub_rows) continue;
+                        for (i64 q = cstart[c]; q < cstart[c + 1]; ++q) {
+                            const int32_t o = crow[q];
+                            if (o == r) continue;
+                            uint32_t h = ((uint32_t)o * 2654435761u) >> 19;  // 13 bits: kSlots
+                            while (key[h] != o && key[h] != -1) h = (h + 1) & (kSlots - 1);
+                            if (key[h] == -1) {
+                                key[h] = o;
+                                used.push_back((int32_t)h);
+                            }
+                            ++hits[h];
+                        }
+                    }
+                    for (int32_t h : used) {
+                        if (hits[h] > most || (hits[h] == most && key[h] < b)) most = hits[h], b = key[h];
+                        key[h] = -1;
+                        hits[h] = 0;
+                    }
+                } else {
+                    touched.clear();
+                    for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) {
+                        const i64 c = elist[e];
+                        if (cstart[c + 1] - cstart[c] > hub_rows) continue;
+                        for (i64 q = cstart[c]; q < cstart[c + 1]; ++q) {
+                            const int32_t o = crow[q];
+                            if (o != r && count[o]++ == 0) touched.push_back(o);
+                        }
+                    }
+                    for (int32_t o : touched) {
+                        if (count[o] > most || (count[o] == most && o < b)) most = count[o], b = o;
+                        count[o] = 0;
+                    }
                 }
                 best[r] = b;
                 shared[r] = most;
