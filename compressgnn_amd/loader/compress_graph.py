@@ -3,6 +3,8 @@
 degrees.  Same fields, constructor and to() as the reference's
 loader/compress_graph.py:6-57; on a GPU it additionally carries the propagation plan
 (int32 index arrays, rows of non-zeros, transposes) that the HIP kernels read."""
+from concurrent.futures import ThreadPoolExecutor
+
 import _paths  # noqa: F401
 import torch
 
@@ -115,13 +117,22 @@ class CompressGraph():
             # rows of the input follow each other and are processed on one XCD), which cuts
             # the misses in the per-XCD L2 caches; results do not depend on the order in the
             # row schedule, and in the nnz schedule only where a long row is cut into runs.
-            def stage(triple):
-                rp, ci, val = triple
+            def ordered(first, second):
+                rp, ci, val = csr_hstack(first, second, V)
                 order = csr_locality_order(rp, ci)
-                rp, ci, val = csr_permute_rows(rp, ci, val, order)
+                return csr_permute_rows(rp, ci, val, order) + (order,)
+
+            def stage(rp, ci, val, order):
                 return rt.DeviceCsr(t(rp), t(ci), t(val), V, V + R, dev, seg, t(order))
 
-            plan.vertex_stage = stage(csr_hstack(host(self.v2v_graph.csr()), host(self.v2r_graph.csr()), V))
-            plan.vertex_stage_t = stage(csr_hstack(host(self.v2v_graph.csc()), host(self.r2v_graph.csc()), V))
+            # The two orders are host work with serial stretches (the host library releases the
+            # interpreter lock while it runs), so they are computed side by side.
+            forward_blocks = (host(self.v2v_graph.csr()), host(self.v2r_graph.csr()))
+            backward_blocks = (host(self.v2v_graph.csc()), host(self.r2v_graph.csc()))
+            with ThreadPoolExecutor(max_workers=2) as pool:
+                forward_job = pool.submit(ordered, *forward_blocks)
+                backward_job = pool.submit(ordered, *backward_blocks)
+                plan.vertex_stage = stage(*forward_job.result())
+                plan.vertex_stage_t = stage(*backward_job.result())
             self._plan = plan
         return self._plan
