@@ -473,9 +473,9 @@ def main():
     plain = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(e2), torch.from_numpy(w), C1_VERTICES,
                          C1_VERTICES, dev)
     pb_f, pb_b = block_bytes(cp, row, C1_VERTICES, F, 0), block_bytes(v2, e2, C1_VERTICES, F, 0)
-    for name in ("rowbalance", "nnzbalance"):
-        f_ms = time_loop(lambda: plain_t.spmm(x, None, name), args.steps, 2, torch)
-        b_ms = time_loop(lambda: plain.spmm(g, None, name), args.steps, 2, torch)
+    for name, forced in (("rowbalance", "row_schedule"), ("nnzbalance", "nnz_schedule")):
+        f_ms = time_loop(lambda: plain_t.spmm(x, None, forced), args.steps, 2, torch)
+        b_ms = time_loop(lambda: plain.spmm(g, None, forced), args.steps, 2, torch)
         detail["plain_csr_%s" % name] = dict(forward_ms=f_ms, backward_ms=b_ms,
                                              forward_GBps=pb_f["bytes"] / (f_ms * 1e-3) / 1e9,
                                              backward_GBps=pb_b["bytes"] / (b_ms * 1e-3) / 1e9,
@@ -490,14 +490,14 @@ def main():
                          C1_VERTICES, dev)
     lb = block_bytes(v2, col_l, C1_VERTICES, F, 0)
     detail["windowed_graph_same_row_lengths"] = {}
-    for name in ("rowbalance", "nnzbalance"):
-        l_ms = time_loop(lambda: local.spmm(x, None, name), args.steps, 2, torch)
+    for name, forced in (("rowbalance", "row_schedule"), ("nnzbalance", "nnz_schedule")):
+        l_ms = time_loop(lambda: local.spmm(x, None, forced), args.steps, 2, torch)
         detail["windowed_graph_same_row_lengths"][name] = dict(ms=l_ms, bytes=lb["bytes"],
                                                                GBps=lb["bytes"] / (l_ms * 1e-3) / 1e9)
     del local
     # parity of the measured configuration: compressed == plain within tolerance
     out, gx = step()
-    ref_out = plain_t.spmm(x, None, "rowbalance")
+    ref_out = plain_t.spmm(x, None, "row_schedule")
     err = (out - ref_out).abs().max().item()
     detail["max_abs_diff_vs_plain_csr"] = err
 

@@ -234,6 +234,15 @@ def csr_transpose(rowptr, col, value, cols):
     return colptr, row, tval
 
 
+def _id_flag(dev):
+    return torch.zeros(1, dtype=torch.int32, device=dev)
+
+
+def _check_id_flag(flag, what, groups):
+    if int(flag.item()) != 0:
+        raise CgnnError("%s: cluster id outside [0, %d)" % (what, groups))
+
+
 def cluster_members(ids, groups):
     """(offsets int32 [groups+1], perm int32 [N], sorted_id int32 [N])."""
     N = ids.numel()
@@ -244,8 +253,10 @@ def cluster_members(ids, groups):
     sorted_id = torch.empty(N, dtype=torch.int32, device=dev)
     need = L.cgnn_cluster_members_workspace_bytes(i64(N), i64(groups))
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    bad = _id_flag(dev)
     check(L.cgnn_cluster_members(i64(N), i64(groups), ptr(ids), ptr(offsets), ptr(perm), ptr(sorted_id),
-                                 ptr(ws), ctypes.c_size_t(need), stream_of(ids)))
+                                 ptr(bad), ptr(ws), ctypes.c_size_t(need), stream_of(ids)))
+    _check_id_flag(bad, "cluster_members", groups)
     return offsets, perm, sorted_id
 
 
@@ -268,8 +279,11 @@ def cluster_mean_backward(grad, ids, counts, members=None):
     F = grad.shape[1]
     dx = torch.empty((N, F), dtype=grad.dtype, device=grad.device)
     perm = None if members is None else members[1]
+    bad = _id_flag(grad.device)
     check(lib().cgnn_cluster_mean_backward(i64(N), i64(F), i64(counts.numel()), dtype_code(grad.dtype),
-                                           ptr(grad), ptr(ids), ptr(counts), ptr(perm), ptr(dx), stream_of(grad)))
+                                           ptr(grad), ptr(ids), ptr(counts), ptr(perm), ptr(dx), ptr(bad),
+                                           stream_of(grad)))
+    _check_id_flag(bad, "cluster_mean_backward", counts.numel())
     return dx
 
 
@@ -278,9 +292,11 @@ def reconstruct(reps, ids, bias=None, relu=False, members=None):
     F = reps.shape[1]
     out = torch.empty((N, F), dtype=reps.dtype, device=reps.device)
     perm = None if members is None else members[1]
+    bad = _id_flag(reps.device)
     check(lib().cgnn_reconstruct(i64(N), i64(F), i64(reps.shape[0]), dtype_code(reps.dtype), ptr(reps),
                                  ptr(ids), ptr(perm), ptr(bias), ctypes.c_int(1 if relu else 0), ptr(out),
-                                 stream_of(reps)))
+                                 ptr(bad), stream_of(reps)))
+    _check_id_flag(bad, "reconstruct", reps.shape[0])
     return out
 
 

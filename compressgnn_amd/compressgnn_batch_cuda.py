@@ -23,7 +23,10 @@ def is_available():
     return torch.cuda.is_available()
 
 
-def compress_csr_batch(vlist, elist, rounds=12, min_pair_frequency=16):
+def compress_csr_batch(vlist, elist, rounds=12, min_pair_frequency=16, release_cache=False):
+    """release_cache=True hands the workspace (about 70 bytes per edge) back to the device
+    afterwards with torch.cuda.empty_cache(), which also flushes whatever else the caller's
+    allocator holds cached: for a preparation script that goes on to build a large model."""
     import torch
     try:
         from compressgnn_amd import abi
@@ -66,7 +69,7 @@ def compress_csr_batch(vlist, elist, rounds=12, min_pair_frequency=16):
         raise RuntimeError(msg)
     R, n = int(summary[0]), int(summary[1])
     result = out_ptr[:V + R + 1].cpu().numpy(), out_col[:n].cpu().numpy(), V, R
-    # the workspace (about 70 bytes per edge) goes back to the device, not into torch's cache
     del dv, de, out_ptr, out_col, ws
-    torch.cuda.empty_cache()
+    if release_cache:
+        torch.cuda.empty_cache()
     return result

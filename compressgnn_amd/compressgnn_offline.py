@@ -278,6 +278,20 @@ def csr_fold_levels(base, levels):
     return nv, ne, nw
 
 
+def csr_fold_levels_bound(base, levels):
+    """Upper bound on the entries of csr_fold_levels(base, levels): the entries before equal
+    columns of a row are merged.  Row sizes only (a float64 per rule, one pass per level), so a
+    deep hierarchy whose folded rows would be huge is seen before anything is built."""
+    size = np.diff(_i64(base[0])).astype(np.float64)
+    for lv, le, _ in levels:
+        lv, le = _i64(lv), _i64(le)
+        if len(le) == 0:
+            continue
+        rows = np.repeat(np.arange(len(lv) - 1), np.diff(lv))
+        size = size + np.bincount(rows, weights=size[le], minlength=len(size))
+    return float(size.sum())
+
+
 def csr_locality_order(vlist, elist):
     """Rows sorted lexicographically by their column lists (int32 [rows])."""
     vlist, elist = _i64(vlist), _i64(elist)

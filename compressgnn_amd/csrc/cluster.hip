@@ -748,6 +748,7 @@ struct GatherArgs {
     const int32_t *__restrict__ perm; // [N] or NULL: order in which the rows are produced
     const T *__restrict__ bias;
     T *__restrict__ out;             // [N x F]
+    int32_t *bad_id;                 // set to 1 when an id lies outside [0, groups), or NULL
     int64_t N, F, groups;
     int32_t relu;
 };
@@ -781,6 +782,12 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
         const int64_t p = first + r < a.N ? first + r : a.N - 1;
         row[r] = a.perm ? (int64_t)a.perm[p] : p;
         g[r] = a.ids[row[r]];
+        // An id from outside the assignment operators may name no row of src: it is moved to the
+        // nearest row that exists, so no access leaves the arrays, and reported through the flag.
+        if (g[r] < 0 || g[r] >= a.groups) {
+            g[r] = g[r] < 0 ? 0 : a.groups - 1;
+            if (a.bad_id) *a.bad_id = 1;  // every writer stores the same value
+        }
     }
     T denom[kGatherRows];
     if constexpr (OP == GATHER_MEAN_GRAD) {
@@ -1027,7 +1034,7 @@ extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int64_t m
 template <typename T, int OP>
 static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, const int64_t *ids,
                         const int32_t *counts, const int32_t *perm, const void *bias, int relu, void *out,
-                        hipStream_t stream) {
+                        int32_t *bad_id, hipStream_t stream) {
     GatherArgs<T> a{};
     a.src = static_cast<const T *>(src);
     a.ids = ids;
@@ -1036,6 +1043,7 @@ static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, c
     a.perm = (F * (int64_t)sizeof(T)) % 128 == 0 ? perm : nullptr;
     a.bias = static_cast<const T *>(bias);
     a.out = static_cast<T *>(out);
+    a.bad_id = bad_id;
     a.N = N;
     a.F = F;
     a.groups = groups;
@@ -1046,27 +1054,28 @@ static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, c
 extern "C" int cgnn_cluster_mean_backward(int64_t N, int64_t F, int64_t groups, int dtype,
                                           const void *grad, const int64_t *ids,
                                           const int32_t *counts, const int32_t *perm, void *dx,
-                                          cgnn_stream_t stream) {
+                                          int32_t *bad_id, cgnn_stream_t stream) {
     CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 1, "cgnn_cluster_mean_backward: bad size");
     if (N == 0 || F == 0) return CGNN_OK;
     CGNN_REQUIRE(grad && ids && counts && dx, "cgnn_cluster_mean_backward: null array");
     if (dtype == CGNN_F32)
-        return gather_typed<float, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, perm, nullptr, 0, dx, stream);
+        return gather_typed<float, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, perm, nullptr, 0, dx, bad_id, stream);
     if (dtype == CGNN_F64)
-        return gather_typed<double, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, perm, nullptr, 0, dx, stream);
+        return gather_typed<double, GATHER_MEAN_GRAD>(N, F, groups, grad, ids, counts, perm, nullptr, 0, dx, bad_id, stream);
     return fail(CGNN_EUNSUPPORTED, "cgnn_cluster_mean_backward: dtype must be f32 or f64");
 }
 
 extern "C" int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
                                 const int64_t *ids, const int32_t *perm, const void *bias, int relu,
-                                void *out, cgnn_stream_t stream) {
+                                void *out, int32_t *bad_id, cgnn_stream_t stream) {
     CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 0, "cgnn_reconstruct: bad size");
+    CGNN_REQUIRE(N == 0 || F == 0 || groups >= 1, "cgnn_reconstruct: rows to reconstruct but no representatives");
     if (N == 0 || F == 0) return CGNN_OK;
     CGNN_REQUIRE(reps && ids && out, "cgnn_reconstruct: null array");
     if (dtype == CGNN_F32)
-        return gather_typed<float, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, relu, out, stream);
+        return gather_typed<float, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, relu, out, bad_id, stream);
     if (dtype == CGNN_F64)
-        return gather_typed<double, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, relu, out, stream);
+        return gather_typed<double, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, relu, out, bad_id, stream);
     return fail(CGNN_EUNSUPPORTED, "cgnn_reconstruct: dtype must be f32 or f64");
 }
 

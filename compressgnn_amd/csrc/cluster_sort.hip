@@ -16,11 +16,19 @@
 namespace cgnn {
 namespace {
 
+// An id outside [0, groups) is filed under the nearest group that exists (the lists then
+// index nothing beyond their arrays) and reported through the flag.
 __global__ void members_keys_kernel(const int64_t *__restrict__ ids, int32_t *__restrict__ keys,
-                                    int32_t *__restrict__ rows, int64_t N) {
+                                    int32_t *__restrict__ rows, int64_t N, int64_t groups,
+                                    int32_t *__restrict__ bad_id) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
          i += (int64_t)gridDim.x * blockDim.x) {
-        keys[i] = (int32_t)ids[i];
+        int64_t id = ids[i];
+        if (id < 0 || id >= groups) {
+            id = id < 0 ? 0 : groups - 1;
+            if (bad_id) *bad_id = 1;  // every writer stores the same value
+        }
+        keys[i] = (int32_t)id;
         rows[i] = (int32_t)i;
     }
 }
@@ -183,7 +191,7 @@ extern "C" size_t cgnn_cluster_members_workspace_bytes(int64_t N, int64_t groups
 }
 
 extern "C" int cgnn_cluster_members(int64_t N, int64_t groups, const int64_t *ids, int32_t *offsets,
-                                    int32_t *perm, int32_t *sorted_id, void *workspace,
+                                    int32_t *perm, int32_t *sorted_id, int32_t *bad_id, void *workspace,
                                     size_t workspace_bytes, cgnn_stream_t stream) {
     CGNN_REQUIRE(N >= 0 && groups >= 1, "cgnn_cluster_members: bad size");
     CGNN_REQUIRE(N < INT32_MAX && groups < INT32_MAX, "cgnn_cluster_members: sizes must be below 2^31");
@@ -203,7 +211,7 @@ extern "C" int cgnn_cluster_members(int64_t N, int64_t groups, const int64_t *id
         int64_t blocks = ceil_div(N, kBlock);
         if (blocks > 8192) blocks = 8192;
         hipLaunchKernelGGL(members_keys_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, ids,
-                           keys, rows, N);
+                           keys, rows, N, groups, bad_id);
         size_t tb = temp_bytes;
         hipError_t e = hipcub::DeviceRadixSort::SortPairs(temp, tb, keys, sorted_id, rows, perm, (int)N,
                                                           0, key_bits(groups), stream);

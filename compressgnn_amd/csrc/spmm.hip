@@ -39,7 +39,6 @@
 // X may alias Y when accumulating (rule levels are updated in place, reference
 // layer/CompressgnnSPMM.py:56-58), so X and Y carry no __restrict__; a row that is
 // written is never gathered in the same launch (levels only read earlier levels).
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -794,22 +793,14 @@ struct Shape {
     int vec, lpr, tiles, grid_y;
 };
 
-int env_int(const char *name) {
-    const char *s = std::getenv(name);
-    return s ? std::atoi(s) : 0;
-}
-
 // Lane layout for a feature width: the widest vector the width and the pointers'
 // alignment allow, then as many lanes as a row needs (power of two, 4..64).
-// CGNN_SPMM_VEC / CGNN_SPMM_LPR (environment, read once) override the choice where the
-// result is a layout that exists; they are for tuning experiments.
 // min_lpr: narrow the vectors (down to single words) while a row would take fewer lanes than
 // this.  The nnz schedule asks for 16: with 4 lanes per run a wave walks 16 runs at once, each
 // with its own row changes (F = 16: 0.106 -> 0.089 ms for the forward vertex stage of the web
 // graph); the row schedule is faster with the widest vectors (0.036 against 0.053 ms).
 template <typename T>
 Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, const void *p3, int min_lpr = 4) {
-    static const int force_vec = env_int("CGNN_SPMM_VEC"), force_lpr = env_int("CGNN_SPMM_LPR");
     auto aligned = [&](size_t bytes) {
         auto ok = [&](const void *p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0; };
         return ok(p0) && ok(p1) && ok(p2) && ok(p3);
@@ -820,14 +811,11 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
         if (F % 4 == 0 && aligned(16)) s.vec = 4;
         else if (F % 2 == 0 && aligned(8)) s.vec = 2;
         while (s.vec > 1 && F / s.vec < min_lpr) s.vec /= 2;
-        if (force_vec == 2 && s.vec == 4) s.vec = 2;
-        if (force_vec == 1) s.vec = 1;
     }
     const int64_t slots = F / s.vec;
     int lpr = pow2_ceil(slots);
     if (lpr < 4) lpr = 4;
     if (lpr > 64) lpr = 64;
-    if (force_lpr >= 4 && force_lpr <= 64 && (force_lpr & (force_lpr - 1)) == 0 && force_lpr < lpr) lpr = force_lpr;
     if (s.vec != 4 || sizeof(T) != 4) {
         // fewer instantiations off the main path: 4, 16 or 64 lanes per row
         lpr = lpr <= 4 ? 4 : (lpr <= 16 ? 16 : 64);
@@ -928,8 +916,7 @@ int resolve_kernel(const cgnn_csr *A, int kernel) {
 }
 
 int seg_len(const cgnn_csr *A) {
-    static const int force_seg = env_int("CGNN_SPMM_SEG");
-    int s = A->seg_nnz > 0 ? A->seg_nnz : (force_seg > 0 ? force_seg : kDefaultSeg);
+    int s = A->seg_nnz > 0 ? A->seg_nnz : kDefaultSeg;
     return (s + kUnroll - 1) / kUnroll * kUnroll;
 }
 

@@ -10,8 +10,8 @@
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
-#include <map>
 #include <memory>
+#include <sstream>
 #include <string>
 #include <tuple>
 #include <vector>
@@ -42,15 +42,29 @@ void require_gpu(const Tensor &t, const char *name) {
 
 // ----------------------------------------------------------------- CSR blocks ----
 
+// Scratch memory of the nnz schedule (the carry rows), grown to the largest request and kept.
+// A block owns one by default; the blocks of a propagation plan share one, since their
+// products follow each other on one stream.  Two streams that run products over the same
+// scratch at the same time would overwrite each other's carries: a caller who does that
+// gives each stream a plan (or a block) of its own.
+struct Scratch {
+    Tensor buf;
+    Tensor get(size_t bytes, const Tensor &like) {
+        if (!buf.defined() || (size_t)buf.numel() < bytes || buf.device() != like.device())
+            buf = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, like.options().dtype(torch::kUInt8));
+        return buf;
+    }
+};
+
 // A CSR block resident on the device in the layout the kernels read (int32 indices,
-// row of every non-zero), with its scratch buffers.  Built once per graph block.
+// row of every non-zero).  Built once per graph block.
 struct DeviceCsr {
     int64_t rows = 0, cols = 0, nnz = 0;
     Tensor rowptr, colidx, rowidx, val;
     Tensor rowmap;  // optional: stored row g is output row rowmap[g]
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
-    std::map<std::tuple<int64_t, int, int>, Tensor> scratch;
+    std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
 
     cgnn_csr view() const {
         cgnn_csr a{};
@@ -70,15 +84,7 @@ struct DeviceCsr {
     Tensor workspace(int64_t F, int dtype, int kernel, size_t *bytes) {
         cgnn_csr a = view();
         *bytes = cgnn_spmm_workspace_bytes(&a, F, dtype, kernel);
-        auto key = std::make_tuple(F, dtype, kernel);
-        auto it = scratch.find(key);
-        if (it == scratch.end() || (size_t)it->second.numel() < *bytes) {
-            Tensor t = torch::empty({(int64_t)std::max<size_t>(*bytes, 1)},
-                                    rowptr.options().dtype(torch::kUInt8));
-            scratch[key] = t;
-            return t;
-        }
-        return it->second;
+        return scratch->get(*bytes, rowptr);
     }
 };
 
@@ -134,16 +140,20 @@ std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Ten
 }
 
 int kernel_of_method(const std::string &method) {
-    // The reference's six GPU method strings (src/runtime/csrc/sparse/cuda/spmm_gpu.cu:27-31)
-    // and its two CPU ones are accepted; "rowbalance*" asks for the row schedule,
-    // "nnzbalance*" for the nnz schedule, "auto" lets the block's row lengths decide.
-    if (method == "auto") return CGNN_SPMM_AUTO;
-    if (method == "rowbalance" || method == "rowbalance_parreduce" || method == "rowbalance_seqreduce" ||
-        method == "rowbalance_rowcache")
-        return CGNN_SPMM_ROW;
-    if (method == "nnzbalance" || method == "nnzbalance_parreduce" || method == "nnzbalance_seqreduce" ||
-        method == "nnzbalance_rowcache")
-        return CGNN_SPMM_NNZ;
+    // The reference's GPU method strings (src/runtime/csrc/sparse/cuda/spmm_gpu.cu:27-31) and
+    // its two CPU ones are accepted.  Its layers pick among them from (nnz, width) alone
+    // (layer/CompressgnnSPMM.py:14-19) and, for instance, ask for "rowbalance_rowcache" on every
+    // large block, power-law in-lists included, where a lane group per row is many times slower
+    // here.  They are therefore hints: the schedule is chosen from the block's row lengths, as
+    // for "auto".  "row_schedule" and "nnz_schedule" are this build's names for a forced
+    // schedule (bit-exact comparisons with a sequential sum, measurements).
+    static const char *const hints[] = {"auto", "rowbalance", "rowbalance_parreduce", "rowbalance_seqreduce",
+                                        "rowbalance_rowcache", "nnzbalance", "nnzbalance_parreduce",
+                                        "nnzbalance_seqreduce", "nnzbalance_rowcache"};
+    for (const char *h : hints)
+        if (method == h) return CGNN_SPMM_AUTO;
+    if (method == "row_schedule") return CGNN_SPMM_ROW;
+    if (method == "nnz_schedule") return CGNN_SPMM_NNZ;
     TORCH_CHECK(false, "Invalid SpMM method: ", method);
 }
 
@@ -250,14 +260,29 @@ struct StageTimer {
 // The device form of a CompressGraph (loader/compress_graph.py:6-43 of the reference):
 // the three vertex/rule blocks, the rule levels and their transposes.
 struct PropagationPlan {
-    std::shared_ptr<DeviceCsr> v2v, v2r, r2v, v2v_t, v2r_t, r2v_t;
+    // rule stage and rule levels, forward and backward
+    std::shared_ptr<DeviceCsr> r2v, v2r_t;
     std::vector<std::shared_ptr<DeviceCsr>> r2r, r2r_t;
     // [v2v | v2r] and [v2v^T | r2v^T]: the vertex stage of forward / backward in one pass
     std::shared_ptr<DeviceCsr> vertex_stage, vertex_stage_t;
+    // the four blocks of the vertex stages on their own: only for the two-launch form
+    // (fuse_final = false); a plan without them holds the graph once
+    std::shared_ptr<DeviceCsr> v2v, v2r, v2v_t, r2v_t;
     int64_t V = 0, R = 0;
     bool fuse_final = true;  // last two stages in one pass (cgnn_spmm_dual)
     int kernel = CGNN_SPMM_AUTO;
+    std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
     StageTimer timer;
+
+    void adopt(const std::shared_ptr<DeviceCsr> &block) {
+        if (block) block->scratch = scratch;
+    }
+    bool fused() const { return fuse_final && vertex_stage && vertex_stage_t; }
+    void require_split_blocks() const {
+        TORCH_CHECK(v2v && v2r && v2v_t && r2v_t,
+                    "this plan holds the fused vertex stages only; the two-launch form needs the v2v, v2r, v2v_t and "
+                    "r2v_t blocks (graph.keep_split_blocks = True before graph.plan())");
+    }
 };
 
 Tensor timed_spmm(PropagationPlan &p, const std::string &stage, DeviceCsr &A, const Tensor &mat,
@@ -269,8 +294,9 @@ Tensor timed_spmm(PropagationPlan &p, const std::string &stage, DeviceCsr &A, co
     return r;
 }
 
-Tensor final_stage(PropagationPlan &p, const std::string &prefix, DeviceCsr *merged, DeviceCsr &from_rules,
-                   const Tensor &rule_x, DeviceCsr &from_vertices, const Tensor &x) {
+Tensor final_stage(PropagationPlan &p, const std::string &prefix, DeviceCsr *merged,
+                   const std::shared_ptr<DeviceCsr> &from_rules, const Tensor &rule_x,
+                   const std::shared_ptr<DeviceCsr> &from_vertices, const Tensor &x) {
     const int64_t F = x.size(1);
     if (p.fuse_final && merged != nullptr) {
         Tensor out = torch::empty({merged->rows, F}, x.options());
@@ -281,14 +307,15 @@ Tensor final_stage(PropagationPlan &p, const std::string &prefix, DeviceCsr *mer
         hipStream_t stream = reinterpret_cast<hipStream_t>(current_stream(x));
         const int id = p.timer.open(prefix + "final", stream);
         cgnn_csr a = merged->view();
-        ok(cgnn_spmm_dual(&a, from_vertices.cols, dtype, x.data_ptr(), rule_x.data_ptr(), out.data_ptr(), F, p.kernel,
+        ok(cgnn_spmm_dual(&a, p.V, dtype, x.data_ptr(), rule_x.data_ptr(), out.data_ptr(), F, p.kernel,
                           ws.data_ptr(), bytes, current_stream(x)),
            "spmm_dual");
         p.timer.close(id, stream);
         return out;
     }
-    Tensor out = timed_spmm(p, prefix + "from_rules", from_rules, rule_x, c10::nullopt);
-    return timed_spmm(p, prefix + "from_vertices", from_vertices, x, out);
+    p.require_split_blocks();
+    Tensor out = timed_spmm(p, prefix + "from_rules", *from_rules, rule_x, c10::nullopt);
+    return timed_spmm(p, prefix + "from_vertices", *from_vertices, x, out);
 }
 
 // layer/CompressgnnSPMM.py:43-62 of the reference.  Stage names: fwd.rules (r2v),
@@ -301,7 +328,7 @@ Tensor propagate_forward(PropagationPlan &p, Tensor x) {
     Tensor rule_out = timed_spmm(p, "fwd.rules", *p.r2v, x, c10::nullopt);
     for (size_t i = 0; i < p.r2r.size(); ++i)
         rule_out = timed_spmm(p, "fwd.level" + std::to_string(i), *p.r2r[i], rule_out, rule_out);
-    return final_stage(p, "fwd.", p.vertex_stage.get(), *p.v2r, rule_out, *p.v2v, x);
+    return final_stage(p, "fwd.", p.vertex_stage.get(), p.v2r, rule_out, p.v2v, x);
 }
 
 // layer/CompressgnnSPMM.py:65-86 (the working branch, lines 80-85).  Stage names as in
@@ -314,40 +341,80 @@ Tensor propagate_backward(PropagationPlan &p, Tensor grad) {
     Tensor rule_g = timed_spmm(p, "bwd.rules", *p.v2r_t, grad, c10::nullopt);
     for (size_t i = p.r2r_t.size(); i-- > 0;)
         rule_g = timed_spmm(p, "bwd.level" + std::to_string(i), *p.r2r_t[i], rule_g, rule_g);
-    return final_stage(p, "bwd.", p.vertex_stage_t.get(), *p.r2v_t, rule_g, *p.v2v_t, grad);
+    return final_stage(p, "bwd.", p.vertex_stage_t.get(), p.r2v_t, rule_g, p.v2v_t, grad);
 }
 
 // ---------------------------------------------------- transformation compression ----
 
-int bucket_size(int64_t bits) {
-    TORCH_CHECK(bits >= 0 && bits <= 30, "Hash bits must be in [0,30]");
-    return 1 << bits;
+// Operand checks of the transformation-compression operators.  Every operator names its
+// operands once, as a row of Operand records, and `expect` reports the first one that does not
+// fit, saying what was asked for and what arrived.
+enum class Role { Features, Ids, Counts, Bias };
+
+struct Operand {
+    Role role;
+    const char *name;
+    const Tensor *tensor;
+};
+
+std::string seen(const Tensor &t) {
+    std::ostringstream os;
+    os << t.scalar_type() << t.sizes() << " on " << t.device() << (t.is_contiguous() ? "" : ", not contiguous");
+    return os.str();
 }
 
-void check_float(const Tensor &x) {
-    TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.is_contiguous(), "Expected contiguous GPU matrix");
-    TORCH_CHECK(x.scalar_type() == torch::kFloat32 || x.scalar_type() == torch::kFloat64,
-                "Only float32 and float64 are supported");
+// `anchor`: the operand whose device (and, for floating operands, precision) the others share.
+void expect(const char *op, const Tensor &anchor, std::initializer_list<Operand> operands) {
+    for (const Operand &o : operands) {
+        const Tensor &t = *o.tensor;
+        bool fits = t.defined() && t.is_cuda() && t.is_contiguous() && t.device() == anchor.device();
+        const char *asked = "";
+        switch (o.role) {
+            case Role::Features:
+                asked = "a contiguous [rows, width] float32 or float64 matrix on the GPU";
+                fits = fits && t.dim() == 2 && (t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kFloat64) &&
+                       t.scalar_type() == anchor.scalar_type();
+                break;
+            case Role::Ids:
+                asked = "a contiguous int64 vector of cluster ids beside the features";
+                fits = fits && t.dim() == 1 && t.scalar_type() == torch::kInt64;
+                break;
+            case Role::Counts:
+                asked = "a contiguous int32 vector with at least the empty cluster 0, beside the features";
+                fits = fits && t.dim() == 1 && t.scalar_type() == torch::kInt32 && t.numel() > 0;
+                break;
+            case Role::Bias:
+                asked = "a contiguous vector of the features' precision, beside the features";
+                fits = fits && t.dim() == 1 && t.scalar_type() == anchor.scalar_type();
+                break;
+        }
+        TORCH_CHECK(fits, op, ": ", o.name, " has to be ", asked, "; it is ", t.defined() ? seen(t) : "undefined");
+    }
 }
-void check_index(const Tensor &index, torch::Device device) {
-    TORCH_CHECK(index.device() == device && index.dim() == 1 && index.is_contiguous() &&
-                    index.scalar_type() == torch::kInt64,
-                "Expected contiguous int64 index on input device");
+
+// Number of hash buckets for `bits` sign bits.
+int64_t buckets_for(const char *op, int64_t bits) {
+    TORCH_CHECK(0 <= bits && bits <= 30, op, ": between 0 and 30 hyperplanes are supported, ", bits, " asked for");
+    return int64_t(1) << bits;
 }
-void check_count(const Tensor &count, torch::Device device) {
-    TORCH_CHECK(count.device() == device && count.dim() == 1 && count.is_contiguous() &&
-                    count.scalar_type() == torch::kInt32 && count.numel() >= 1,
-                "Expected nonempty int32 counts on input device");
+
+// The hyperplanes of an assignment: one column per sign bit, one row per input feature.
+void expect_planes(const char *op, const Tensor &input, const Tensor &planes, int64_t bits) {
+    expect(op, input, {{Role::Features, "input", &input}, {Role::Features, "hyperplanes", &planes}});
+    TORCH_CHECK(planes.size(0) == input.size(1) && planes.size(1) == bits, op, ": ", bits, " hyperplanes over ",
+                input.size(1), " features make a [", input.size(1), ", ", bits, "] matrix, not ", planes.sizes());
+    TORCH_CHECK(input.size(0) < INT_MAX, op, ": ", input.size(0), " rows do not fit the int32 cluster sizes");
 }
 
 // cluster_workspace_cuda (src/runtime/csrc/cluster/cuda/cluster_kernel.cu:111-117):
 // [bucket counts int32[2^bits], prefix int32[2^bits], scan scratch uint8[...]].
 std::vector<Tensor> cluster_workspace(Tensor input, int64_t bits) {
-    check_float(input);
+    const char *op = "cluster_workspace";
+    expect(op, input, {{Role::Features, "input", &input}});
+    const int64_t buckets = buckets_for(op, bits);
     c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
-    const int n = bucket_size(bits);
     auto ints = input.options().dtype(torch::kInt32);
-    return {torch::empty({n}, ints), torch::empty({n}, ints),
+    return {torch::empty({buckets}, ints), torch::empty({buckets}, ints),
             torch::empty({(int64_t)cgnn_lsh_scan_workspace_bytes((int)bits)}, input.options().dtype(torch::kUInt8))};
 }
 
@@ -361,14 +428,10 @@ std::vector<Tensor> cluster_workspace(Tensor input, int64_t bits) {
 // comes last and only trims the views.
 std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(Tensor input, Tensor planes,
                                                                                 int64_t bits) {
-    check_float(input);
-    check_float(planes);
+    const char *op = "cluster_assign";
+    const int64_t buckets = buckets_for(op, bits);
+    expect_planes(op, input, planes, bits);
     c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
-    const int n = bucket_size(bits);
-    TORCH_CHECK(planes.device() == input.device() && planes.scalar_type() == input.scalar_type() &&
-                    planes.size(0) == input.size(1) && planes.size(1) == bits,
-                "Hash plane shape/device/dtype mismatch");
-    TORCH_CHECK(input.size(0) < INT_MAX, "Node count exceeds int32 capacity");
     const int64_t N = input.size(0);
     auto ints = input.options().dtype(torch::kInt32);
     Tensor ids = torch::empty({N}, input.options().dtype(torch::kInt64));
@@ -376,7 +439,7 @@ std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(
     auto host_scalar = [](int64_t v) { return torch::full({1}, v, torch::TensorOptions().dtype(torch::kInt64)); };
     if (N == 0)
         return {ids, torch::zeros({1}, ints), 0, {torch::zeros({2}, ints), perm, sorted_id, host_scalar(0)}};
-    const int64_t cap = std::min<int64_t>(N, n);
+    const int64_t cap = std::min<int64_t>(N, buckets);
     Tensor raw = torch::empty({N}, ints);
     Tensor offsets = torch::empty({cap + 2}, ints), counts = torch::empty({cap + 1}, ints);
     Tensor summary_dev = torch::empty({2}, ints);  // number of groups, largest group
@@ -396,27 +459,25 @@ std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(
             {offsets.narrow(0, 0, active + 2), perm, sorted_id, host_scalar(summary.data_ptr<int32_t>()[1])}};
 }
 
-// cluster_assign_cuda (cluster_kernel.cu:118-153).  The workspace of cluster_workspace is
-// checked as there; the grouping itself no longer needs bucket counters.
+// cluster_assign_cuda (cluster_kernel.cu:118-153).  The three tensors of cluster_workspace
+// are accepted, and must be what cluster_workspace returns for these arguments; the grouping
+// itself sorts the codes and no longer touches bucket counters.
 std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, int64_t bits,
                                                    std::vector<Tensor> workspace) {
-    check_float(input);
-    check_float(planes);
-    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
-    const int n = bucket_size(bits);
-    TORCH_CHECK(planes.device() == input.device() && planes.scalar_type() == input.scalar_type() &&
-                    planes.size(0) == input.size(1) && planes.size(1) == bits,
-                "Hash plane shape/device/dtype mismatch");
-    TORCH_CHECK(input.size(0) <= INT_MAX, "Node count exceeds int32 bucket count capacity");
-    TORCH_CHECK(workspace.size() == 3, "Expected bucket, prefix and scan workspaces");
-    for (int i = 0; i < 3; ++i)
-        TORCH_CHECK(workspace[i].device() == input.device() && workspace[i].dim() == 1 && workspace[i].is_contiguous(),
-                    "Workspace device/shape mismatch");
-    const size_t scan_bytes = cgnn_lsh_scan_workspace_bytes((int)bits);
-    TORCH_CHECK(workspace[0].scalar_type() == torch::kInt32 && workspace[1].scalar_type() == torch::kInt32 &&
-                    workspace[0].numel() == n && workspace[1].numel() == n &&
-                    workspace[2].scalar_type() == torch::kUInt8 && (size_t)workspace[2].numel() >= scan_bytes,
-                "Workspace dtype/capacity mismatch");
+    const char *op = "cluster_assign";
+    const int64_t buckets = buckets_for(op, bits);
+    expect_planes(op, input, planes, bits);
+    TORCH_CHECK(workspace.size() == 3, op, ": the workspace is the three tensors of cluster_workspace, ", workspace.size(),
+                " given");
+    const int64_t need[3] = {buckets, buckets, (int64_t)cgnn_lsh_scan_workspace_bytes((int)bits)};
+    const torch::ScalarType kind[3] = {torch::kInt32, torch::kInt32, torch::kUInt8};
+    for (int i = 0; i < 3; ++i) {
+        const Tensor &w = workspace[i];
+        const bool fits = w.defined() && w.device() == input.device() && w.dim() == 1 && w.is_contiguous() &&
+                          w.scalar_type() == kind[i] && (i < 2 ? w.numel() == need[i] : w.numel() >= need[i]);
+        TORCH_CHECK(fits, op, ": workspace[", i, "] has to be ", kind[i], "[", need[i], "] beside the input; it is ",
+                    w.defined() ? seen(w) : "undefined");
+    }
     auto grouped = cluster_assign_members(input, planes, bits);
     return {std::get<0>(grouped), std::get<1>(grouped), std::get<2>(grouped)};
 }
@@ -424,52 +485,68 @@ std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, 
 // cluster_forward (src/runtime/csrc/cluster/cluster.cpp:12-30): int32 ids and the
 // number of active buckets.
 std::tuple<Tensor, int64_t> cluster_forward(Tensor input, Tensor random_vectors, int64_t param_h) {
-    TORCH_CHECK(input.dim() == 2 && random_vectors.dim() == 2 && input.is_contiguous() && random_vectors.is_contiguous(),
-                "Expected contiguous matrices");
-    TORCH_CHECK(param_h >= 0 && param_h <= 30 && random_vectors.size(0) == input.size(1) && random_vectors.size(1) == param_h,
-                "Invalid hash plane shape/bits");
-    TORCH_CHECK(input.device() == random_vectors.device() && input.scalar_type() == random_vectors.scalar_type(),
-                "Hash device/dtype mismatch");
-    TORCH_CHECK(input.scalar_type() == torch::kFloat32 || input.scalar_type() == torch::kFloat64,
-                "Expected float32/float64 features");
     require_gpu(input, "input");
-    auto result = cluster_assign(input, random_vectors, param_h, cluster_workspace(input, param_h));
-    return {std::get<0>(result).to(torch::kInt32), std::get<2>(result)};
+    auto grouped = cluster_assign_members(input, random_vectors, param_h);
+    return {std::get<0>(grouped).to(torch::kInt32), std::get<2>(grouped)};
 }
+
+// One int32 on the device that the kernels set when they meet a cluster id that names no
+// cluster; `raise` reads it (the only host read of these operators, made only for index
+// tensors that do not come with member lists of this library's own making).
+struct IdFlag {
+    Tensor flag;
+    explicit IdFlag(const Tensor &like) : flag(torch::zeros({1}, like.options().dtype(torch::kInt32))) {}
+    int32_t *ptr() { return flag.data_ptr<int32_t>(); }
+    void raise(const char *op, int64_t groups) {
+        TORCH_CHECK(flag.item<int32_t>() == 0, op, ": the index holds a cluster id outside [0, ", groups, ")");
+    }
+};
 
 // Member lists of `groups` clusters: [offsets int32[groups+1], perm int32[N], sorted_id int32[N]].
 std::vector<Tensor> cluster_members(Tensor index, int64_t groups) {
-    TORCH_CHECK(index.is_cuda(), "index must be a GPU tensor");
-    check_index(index, index.device());
-    TORCH_CHECK(groups >= 1, "groups must be positive");
+    const char *op = "cluster_members";
+    require_gpu(index, "index");
+    expect(op, index, {{Role::Ids, "index", &index}});
+    TORCH_CHECK(groups >= 1, op, ": at least the empty cluster 0 is needed, groups = ", groups);
     c10::hip::HIPGuardMasqueradingAsCUDA guard(index.device());
     const int64_t N = index.numel();
     auto i32 = index.options().dtype(torch::kInt32);
     Tensor offsets = torch::empty({groups + 1}, i32), perm = torch::empty({N}, i32), sorted = torch::empty({N}, i32);
     const size_t bytes = cgnn_cluster_members_workspace_bytes(N, groups);
     Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, index.options().dtype(torch::kUInt8));
+    IdFlag bad(index);
     ok(cgnn_cluster_members(N, groups, N ? index.data_ptr<int64_t>() : nullptr, offsets.data_ptr<int32_t>(),
-                            N ? perm.data_ptr<int32_t>() : nullptr, N ? sorted.data_ptr<int32_t>() : nullptr,
+                            N ? perm.data_ptr<int32_t>() : nullptr, N ? sorted.data_ptr<int32_t>() : nullptr, bad.ptr(),
                             ws.data_ptr(), bytes, current_stream(index)),
-       "cluster_members");
+       op);
+    bad.raise(op, groups);
     return {offsets, perm, sorted};
 }
 
-std::vector<Tensor> members_or_build(const c10::optional<std::vector<Tensor>> &members, const Tensor &index,
-                                     int64_t groups) {
-    if (members.has_value() && !members->empty()) {
-        const auto &m = *members;
-        // an optional fourth entry: a host int64 scalar with the size of the largest group
-        TORCH_CHECK((m.size() == 3 || (m.size() == 4 && !m[3].is_cuda() && m[3].numel() == 1 &&
-                                       m[3].scalar_type() == torch::kInt64)) &&
-                        m[0].numel() == groups + 1 && m[1].numel() == index.numel() &&
-                        m[2].numel() == index.numel() && m[0].scalar_type() == torch::kInt32 &&
-                        m[1].scalar_type() == torch::kInt32 && m[2].scalar_type() == torch::kInt32 &&
-                        m[0].device() == index.device(),
-                    "member lists do not match index/groups");
-        return m;
-    }
-    return cluster_members(index, groups);
+// Member lists handed in by the caller ([offsets, perm, sorted_id] and optionally a host int64
+// scalar with the size of the largest group), checked against the index they belong to.
+bool has_members(const c10::optional<std::vector<Tensor>> &members) { return members.has_value() && !members->empty(); }
+
+void expect_members(const char *op, const std::vector<Tensor> &m, const Tensor &index, int64_t groups) {
+    TORCH_CHECK(m.size() == 3 || m.size() == 4, op, ": member lists are [offsets, perm, sorted_id] (+ largest group), ",
+                m.size(), " tensors given");
+    const int64_t want[3] = {groups + 1, index.numel(), index.numel()};
+    const char *names[3] = {"offsets", "perm", "sorted_id"};
+    for (int i = 0; i < 3; ++i)
+        TORCH_CHECK(m[i].defined() && m[i].scalar_type() == torch::kInt32 && m[i].device() == index.device() &&
+                        m[i].is_contiguous() && (groups < 0 && i == 0 ? true : m[i].numel() == want[i]),
+                    op, ": member list '", names[i], "' has to be int32[", want[i], "] beside the index; it is ",
+                    m[i].defined() ? seen(m[i]) : "undefined");
+    if (m.size() == 4)
+        TORCH_CHECK(!m[3].is_cuda() && m[3].numel() == 1 && m[3].scalar_type() == torch::kInt64, op,
+                    ": the fourth member tensor is a host int64 scalar (size of the largest group)");
+}
+
+std::vector<Tensor> members_or_build(const char *op, const c10::optional<std::vector<Tensor>> &members,
+                                     const Tensor &index, int64_t groups) {
+    if (!has_members(members)) return cluster_members(index, groups);
+    expect_members(op, *members, index, groups);
+    return *members;
 }
 
 int64_t largest_group(const std::vector<Tensor> &m) { return m.size() == 4 ? m[3].item<int64_t>() : 0; }
@@ -477,93 +554,94 @@ int64_t largest_group(const std::vector<Tensor> &m) { return m.size() == 4 ? m[3
 // cluster_mean_cuda (cluster_kernel.cu:158-170).  `members` (from cluster_members, for
 // the same index) avoids rebuilding the member lists on every call.
 Tensor cluster_mean(Tensor input, Tensor index, Tensor count, c10::optional<std::vector<Tensor>> members) {
-    check_float(input);
-    check_index(index, input.device());
-    check_count(count, input.device());
-    TORCH_CHECK(index.numel() == input.size(0), "Input/index length mismatch");
+    const char *op = "cluster_mean";
+    expect(op, input, {{Role::Features, "input", &input}, {Role::Ids, "index", &index}, {Role::Counts, "count", &count}});
+    TORCH_CHECK(index.numel() == input.size(0), op, ": ", input.size(0), " rows but ", index.numel(), " cluster ids");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     const int64_t N = input.size(0), F = input.size(1), groups = count.numel();
     if (input.numel() == 0) return torch::zeros({groups, F}, input.options());
-    auto m = members_or_build(members, index, groups);
+    auto m = members_or_build(op, members, index, groups);
     Tensor out = torch::empty({groups, F}, input.options());
     const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(input));
     Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, input.options().dtype(torch::kUInt8));
     ok(cgnn_cluster_mean(N, F, groups, largest_group(m), dtype_code(input), input.data_ptr(), m[0].data_ptr<int32_t>(),
                          m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(), count.data_ptr<int32_t>(), out.data_ptr(),
                          ws.data_ptr(), bytes, current_stream(input)),
-       "cluster_mean");
+       op);
     return out;
+}
+
+// The order in which a gather produces its rows: the member list `perm` when the caller has one.
+// An index that comes without member lists is an index from outside the assignment operators,
+// and its ids are checked (one host read).
+const int32_t *production_order(const char *op, const c10::optional<std::vector<Tensor>> &members, const Tensor &index) {
+    if (!has_members(members)) return nullptr;
+    expect_members(op, *members, index, -1);
+    return (*members)[1].data_ptr<int32_t>();
 }
 
 // cluster_mean_backward_cuda (cluster_kernel.cu:171-181).
 Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count, c10::optional<std::vector<Tensor>> members) {
-    check_float(grad);
-    check_index(index, grad.device());
-    check_count(count, grad.device());
-    TORCH_CHECK(grad.size(0) == count.numel(), "Gradient/count shape mismatch");
+    const char *op = "cluster_mean_backward";
+    expect(op, grad, {{Role::Features, "grad", &grad}, {Role::Ids, "index", &index}, {Role::Counts, "count", &count}});
+    TORCH_CHECK(grad.size(0) == count.numel(), op, ": ", grad.size(0), " gradient rows for ", count.numel(), " clusters");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
     Tensor out = torch::empty({index.numel(), grad.size(1)}, grad.options());
     if (out.numel() == 0) return out;
-    const int32_t *perm = nullptr;
-    if (members.has_value() && !members->empty()) {
-        TORCH_CHECK(members->size() >= 3 && (*members)[1].numel() == index.numel() &&
-                        (*members)[1].scalar_type() == torch::kInt32 && (*members)[1].device() == index.device(),
-                    "member lists do not match index");
-        perm = (*members)[1].data_ptr<int32_t>();
-    }
+    const int32_t *perm = production_order(op, members, index);
+    c10::optional<IdFlag> bad;
+    if (perm == nullptr) bad.emplace(index);
     ok(cgnn_cluster_mean_backward(index.numel(), grad.size(1), count.numel(), dtype_code(grad), grad.data_ptr(),
                                   index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), perm, out.data_ptr(),
-                                  current_stream(grad)),
-       "cluster_mean_backward");
+                                  bad ? bad->ptr() : nullptr, current_stream(grad)),
+       op);
+    if (bad) bad->raise(op, count.numel());
     return out;
 }
 
 // cluster_reconstruct_cuda (cluster_kernel.cu:182-195).
 Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias, bool relu,
                            c10::optional<std::vector<Tensor>> members) {
-    check_float(reps);
-    check_index(index, reps.device());
-    if (bias.has_value())
-        TORCH_CHECK(bias->device() == reps.device() && bias->scalar_type() == reps.scalar_type() && bias->dim() == 1 &&
-                        bias->numel() == reps.size(1) && bias->is_contiguous(),
-                    "Invalid reconstruction bias");
+    const char *op = "cluster_reconstruct";
+    expect(op, reps, {{Role::Features, "representatives", &reps}, {Role::Ids, "index", &index}});
+    if (bias.has_value()) {
+        expect(op, reps, {{Role::Bias, "bias", &*bias}});
+        TORCH_CHECK(bias->numel() == reps.size(1), op, ": a bias of ", bias->numel(), " entries for rows of ", reps.size(1));
+    }
+    TORCH_CHECK(index.numel() == 0 || reps.size(0) > 0, op, ": rows to reconstruct but no representatives");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(reps.device());
     Tensor out = torch::empty({index.numel(), reps.size(1)}, reps.options());
     if (out.numel() == 0) return out;
-    const int32_t *perm = nullptr;
-    if (members.has_value() && !members->empty()) {
-        TORCH_CHECK(members->size() >= 3 && (*members)[1].numel() == index.numel() &&
-                        (*members)[1].scalar_type() == torch::kInt32 && (*members)[1].device() == index.device(),
-                    "member lists do not match index");
-        perm = (*members)[1].data_ptr<int32_t>();
-    }
+    const int32_t *perm = production_order(op, members, index);
+    c10::optional<IdFlag> bad;
+    if (perm == nullptr) bad.emplace(index);
     ok(cgnn_reconstruct(index.numel(), reps.size(1), reps.size(0), dtype_code(reps), reps.data_ptr(),
                         index.data_ptr<int64_t>(), perm, bias.has_value() ? bias->data_ptr() : nullptr, relu ? 1 : 0,
-                        out.data_ptr(), current_stream(reps)),
-       "cluster_reconstruct");
+                        out.data_ptr(), bad ? bad->ptr() : nullptr, current_stream(reps)),
+       op);
+    if (bad) bad->raise(op, reps.size(0));
     return out;
 }
 
 // cluster_reconstruct_backward_cuda (cluster_kernel.cu:196-208).
 Tensor cluster_reconstruct_backward(Tensor grad, Tensor index, Tensor output, int64_t groups, bool relu,
                                     c10::optional<std::vector<Tensor>> members) {
-    check_float(grad);
-    check_index(index, grad.device());
-    check_float(output);
-    TORCH_CHECK(groups >= 0 && output.sizes() == grad.sizes() && output.device() == grad.device() &&
-                    output.scalar_type() == grad.scalar_type() && index.numel() == grad.size(0),
-                "Invalid reconstruction gradient");
+    const char *op = "cluster_reconstruct_backward";
+    expect(op, grad, {{Role::Features, "grad", &grad}, {Role::Ids, "index", &index}, {Role::Features, "output", &output}});
+    TORCH_CHECK(groups >= 0, op, ": groups = ", groups);
+    TORCH_CHECK(output.sizes() == grad.sizes(), op, ": the saved output is ", output.sizes(), ", the gradient ", grad.sizes());
+    TORCH_CHECK(index.numel() == grad.size(0), op, ": ", grad.size(0), " rows but ", index.numel(), " cluster ids");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
     const int64_t N = grad.size(0), F = grad.size(1);
     if (grad.numel() == 0 || groups == 0) return torch::zeros({groups, F}, grad.options());
-    auto m = members_or_build(members, index, groups);
+    auto m = members_or_build(op, members, index, groups);
     Tensor out = torch::empty({groups, F}, grad.options());
     const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(grad));
     Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, grad.options().dtype(torch::kUInt8));
     ok(cgnn_reconstruct_backward(N, F, groups, largest_group(m), dtype_code(grad), grad.data_ptr(), output.data_ptr(),
                                  m[0].data_ptr<int32_t>(), m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(),
                                  relu ? 1 : 0, out.data_ptr(), ws.data_ptr(), bytes, current_stream(grad)),
-       "cluster_reconstruct_backward");
+       op);
     return out;
 }
 
@@ -654,22 +732,48 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
              },
              py::arg("mat"), py::arg("out") = py::none(), py::arg("method") = "auto");
     py::class_<PropagationPlan, std::shared_ptr<PropagationPlan>>(m, "PropagationPlan")
-        .def(py::init([](std::shared_ptr<DeviceCsr> v2v, std::shared_ptr<DeviceCsr> v2r, std::shared_ptr<DeviceCsr> r2v,
-                         std::vector<std::shared_ptr<DeviceCsr>> r2r, std::shared_ptr<DeviceCsr> v2v_t,
-                         std::shared_ptr<DeviceCsr> v2r_t, std::shared_ptr<DeviceCsr> r2v_t,
-                         std::vector<std::shared_ptr<DeviceCsr>> r2r_t) {
+        .def(py::init([](int64_t V, int64_t R, std::shared_ptr<DeviceCsr> r2v, std::vector<std::shared_ptr<DeviceCsr>> r2r,
+                         std::shared_ptr<DeviceCsr> v2r_t, std::vector<std::shared_ptr<DeviceCsr>> r2r_t) {
                  auto p = std::make_shared<PropagationPlan>();
-                 p->v2v = v2v; p->v2r = v2r; p->r2v = r2v; p->r2r = r2r;
-                 p->v2v_t = v2v_t; p->v2r_t = v2r_t; p->r2v_t = r2v_t; p->r2r_t = r2r_t;
-                 p->V = v2v->rows; p->R = r2v->rows;
+                 TORCH_CHECK(r2v && v2r_t, "the rule stages r2v and v2r_t are required");
                  TORCH_CHECK(r2r.size() == r2r_t.size(), "levels and transposed levels differ in number");
+                 TORCH_CHECK(r2v->rows == R && r2v->cols == V && v2r_t->rows == R && v2r_t->cols == V,
+                             "the rule stages must be [rule_cnt, vertex_cnt]");
+                 p->V = V; p->R = R;
+                 p->r2v = r2v; p->r2r = r2r; p->v2r_t = v2r_t; p->r2r_t = r2r_t;
+                 p->adopt(r2v); p->adopt(v2r_t);
+                 for (auto &b : r2r) p->adopt(b);
+                 for (auto &b : r2r_t) p->adopt(b);
                  return p;
-             }))
-        .def_readwrite("fuse_final", &PropagationPlan::fuse_final)
-        .def_readwrite("vertex_stage", &PropagationPlan::vertex_stage)
-        .def_readwrite("vertex_stage_t", &PropagationPlan::vertex_stage_t)
+             }),
+             py::arg("vertex_cnt"), py::arg("rule_cnt"), py::arg("r2v"), py::arg("r2r"), py::arg("v2r_t"), py::arg("r2r_t"))
+        .def("set_vertex_stages",
+             [](PropagationPlan &p, std::shared_ptr<DeviceCsr> fwd, std::shared_ptr<DeviceCsr> bwd) {
+                 TORCH_CHECK(fwd && bwd && fwd->rows == p.V && bwd->rows == p.V && fwd->cols == p.V + p.R &&
+                                 bwd->cols == p.V + p.R,
+                             "a vertex stage is [vertex_cnt, vertex_cnt + rule_cnt]");
+                 p.vertex_stage = fwd; p.vertex_stage_t = bwd;
+                 p.adopt(fwd); p.adopt(bwd);
+             })
+        .def("set_split_blocks",
+             [](PropagationPlan &p, std::shared_ptr<DeviceCsr> v2v, std::shared_ptr<DeviceCsr> v2r,
+                std::shared_ptr<DeviceCsr> v2v_t, std::shared_ptr<DeviceCsr> r2v_t) {
+                 p.v2v = v2v; p.v2r = v2r; p.v2v_t = v2v_t; p.r2v_t = r2v_t;
+                 p.adopt(v2v); p.adopt(v2r); p.adopt(v2v_t); p.adopt(r2v_t);
+                 p.require_split_blocks();
+             })
+        .def_property("fuse_final", [](PropagationPlan &p) { return p.fuse_final; },
+                      [](PropagationPlan &p, bool fuse) {
+                          if (!fuse) p.require_split_blocks();
+                          else TORCH_CHECK(p.vertex_stage && p.vertex_stage_t, "this plan has no fused vertex stages");
+                          p.fuse_final = fuse;
+                      })
+        .def_readonly("vertex_stage", &PropagationPlan::vertex_stage)
+        .def_readonly("vertex_stage_t", &PropagationPlan::vertex_stage_t)
+        .def_property_readonly("scratch_bytes",
+                               [](PropagationPlan &p) { return p.scratch->buf.defined() ? p.scratch->buf.numel() : 0; })
         .def_property("method",
-                      [](PropagationPlan &p) { return p.kernel == CGNN_SPMM_ROW ? "rowbalance" : p.kernel == CGNN_SPMM_NNZ ? "nnzbalance" : "auto"; },
+                      [](PropagationPlan &p) { return p.kernel == CGNN_SPMM_ROW ? "row_schedule" : p.kernel == CGNN_SPMM_NNZ ? "nnz_schedule" : "auto"; },
                       [](PropagationPlan &p, std::string mth) { p.kernel = kernel_of_method(mth); })
         .def_property("timed_stages", [](PropagationPlan &p) { return p.timer.timed; },
                       [](PropagationPlan &p, std::vector<std::string> names) { p.timer.timed = names; })

@@ -6,8 +6,10 @@ gathers from x, phase k >= 1 from out, every phase adds weight * feature[src] in
 out[dst]; the result is out[:V].  Here every phase is one CSR product of the HIP kernels:
 the edges of a phase are grouped by destination once (stable, so a destination sums its
 messages in edge order), and the gradient runs the transposed phases in reverse order.
-A source of phase k receives nothing in phase k, which is what makes the in-place
-products valid.
+In the phases the loader makes, a source of phase k receives nothing in phase k, so the
+product of a phase k >= 1 accumulates in place.  A phase list from elsewhere may break that;
+such a phase (found when the plan is built, on the host) runs as a fresh product followed by
+an addition, which is what the reference's gather-then-scatter computes for any phase list.
 """
 import _paths  # noqa: F401
 import numpy as np
@@ -32,6 +34,7 @@ class CooPhasePlan:
             raise RuntimeError("multi-phase propagation runs on the GPU only: move the data to a GPU")
         self.device = device
         self.forward_blocks, self.backward_blocks = [], []
+        self.in_place = []  # per phase: no node is both a source and a destination of the phase
         # keeps the tensors (and so their addresses) alive for as long as the plan is cached
         self.sources = (list(edge_index), None if edge_weight is None else list(edge_weight))
         t = torch.from_numpy
@@ -49,6 +52,9 @@ class CooPhasePlan:
             rows_back = cols
             if src.size and (src.min() < 0 or src.max() >= cols or dst.min() < 0 or dst.max() >= total):
                 raise ValueError("phase %d: node id out of range" % k)
+            is_src = np.zeros(total, bool)
+            is_src[src] = True
+            self.in_place.append(not bool(is_src[dst].any()))
             # by source (stable): the transposed block used by the gradient
             by_src = np.argsort(src, kind="stable")
             sp = np.zeros(rows_back + 1, np.int64)
@@ -66,8 +72,8 @@ class CooPhasePlan:
         if x.dim() != 2 or x.size(0) != self.V:
             raise ValueError("x must be [vertex_cnt, F]")
         out = self.forward_blocks[0].spmm(x)
-        for block in self.forward_blocks[1:]:
-            out = block.spmm(out, out)
+        for block, in_place in zip(self.forward_blocks[1:], self.in_place[1:]):
+            out = block.spmm(out, out) if in_place else out + block.spmm(out)
         return out[:self.V]
 
     def backward(self, grad):
@@ -76,8 +82,8 @@ class CooPhasePlan:
             full = grad if self.R == 0 else torch.cat([grad, grad.new_zeros((self.R, grad.size(1)))])
             return self.backward_blocks[0].spmm(full)
         full = torch.cat([grad, grad.new_zeros((self.R, grad.size(1)))])
-        for block in reversed(self.backward_blocks[1:]):
-            full = block.spmm(full, full)
+        for block, in_place in zip(reversed(self.backward_blocks[1:]), reversed(self.in_place[1:])):
+            full = block.spmm(full, full) if in_place else full + block.spmm(full)
         return self.backward_blocks[0].spmm(full)
 
 

@@ -8,7 +8,7 @@ from concurrent.futures import ThreadPoolExecutor
 import _paths  # noqa: F401
 import torch
 
-from compressgnn_offline import (csr_fold_levels, csr_hstack, csr_locality_order, csr_permute_rows, gen_degree,
+from compressgnn_offline import (csr_fold_levels, csr_fold_levels_bound, csr_hstack, csr_locality_order, csr_permute_rows, gen_degree,
                                  hybird_partition, topo_partition)
 from sparse_csr import SparseCSR
 
@@ -37,6 +37,9 @@ class CompressGraph():
         # backward, instead of one more launch per level (the same sums in another order).
         # Set to False before plan() for the launch-per-level form of the reference.
         self.fold_levels = True
+        self.levels_folded = False       # what plan() decided
+        self.keep_split_blocks = False   # plan(): also build the four vertex-stage blocks on their own
+        self.keep_device_blocks = False  # plan(): leave the int64 blocks on the device
         self._plan = None
 
     def __repr__(self):
@@ -75,6 +78,29 @@ class CompressGraph():
     def device(self):
         return self.v2v_graph.device
 
+    # Folding the levels multiplies out the rule hierarchy: a rule row grows to all the vertices
+    # it stands for, which a deep hierarchy can make exponentially many.  The levels are folded
+    # only while the folded rule stage stays within this multiple of the entries of the blocks
+    # it replaces (r2v or v2r plus the levels) and the hierarchy is no deeper than max_fold_depth;
+    # beyond that the plan keeps one launch per level, the reference's form.
+    max_fold_growth = 4.0
+    max_fold_depth = 16
+
+    def _fold_plan(self, host):
+        """(forward base, forward levels, backward base, backward levels) on the host when the
+        levels are to be folded into the rule stage, else None."""
+        if not getattr(self, "fold_levels", True) or self.step == 0:
+            return None
+        if self.step > self.max_fold_depth:
+            return None
+        fwd_base, fwd_levels = host(self.r2v_graph.csr()), [host(g.csr()) for g in self.r2r_graph]
+        bwd_base, bwd_levels = host(self.v2r_graph.csc()), [host(g.csc()) for g in reversed(self.r2r_graph)]
+        for base, levels in ((fwd_base, fwd_levels), (bwd_base, bwd_levels)):
+            stored = len(base[1]) + sum(len(lv[1]) for lv in levels)
+            if csr_fold_levels_bound(base, levels) > self.max_fold_growth * max(stored, 1):
+                return None
+        return fwd_base, fwd_levels, bwd_base, bwd_levels
+
     def plan(self):
         """The device-side propagation plan (built on first use after to(device))."""
         if self._plan is None:
@@ -98,20 +124,22 @@ class CompressGraph():
             V, R = self.vertex_cnt, self.rule_cnt
             host = lambda triple: tuple(t.cpu().numpy() for t in triple)
             t = torch.from_numpy
-            if getattr(self, "fold_levels", True) and self.step > 0:
+            folded = self._fold_plan(host)
+            self.levels_folded = folded is not None
+            if folded is not None:
                 # forward: rule_out = (I + L_last) ... (I + L_0) r2v x; backward, with the
                 # transposed levels in reverse order: rule_g = (I + L_0^T) ... (I + L_last^T) v2r^T g
-                rp, ci, val = csr_fold_levels(host(self.r2v_graph.csr()), [host(g.csr()) for g in self.r2r_graph])
+                rp, ci, val = csr_fold_levels(folded[0], folded[1])
                 rules_fwd = rt.DeviceCsr(t(rp), t(ci), t(val), R, V, dev, seg)
-                rp, ci, val = csr_fold_levels(host(self.v2r_graph.csc()),
-                                              [host(g.csc()) for g in reversed(self.r2r_graph)])
+                rp, ci, val = csr_fold_levels(folded[2], folded[3])
                 rules_bwd = rt.DeviceCsr(t(rp), t(ci), t(val), R, V, dev, seg)
-                plan = rt.PropagationPlan(fwd(self.v2v_graph), fwd(self.v2r_graph), rules_fwd, [],
-                                          bwd(self.v2v_graph), rules_bwd, bwd(self.r2v_graph), [])
+                plan = rt.PropagationPlan(V, R, rules_fwd, [], rules_bwd, [])
             else:
-                plan = rt.PropagationPlan(
-                    fwd(self.v2v_graph), fwd(self.v2r_graph), fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
-                    bwd(self.v2v_graph), bwd(self.v2r_graph), bwd(self.r2v_graph), [bwd(g) for g in self.r2r_graph])
+                plan = rt.PropagationPlan(V, R, fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
+                                          bwd(self.v2r_graph), [bwd(g) for g in self.r2r_graph])
+            if getattr(self, "keep_split_blocks", False):
+                # the vertex stages as two launches each (plan.fuse_final = False)
+                plan.set_split_blocks(fwd(self.v2v_graph), fwd(self.v2r_graph), bwd(self.v2v_graph), bwd(self.r2v_graph))
             # the vertex stage reads [v2v | v2r] (forward) and [v2v^T | r2v^T] (backward) in one pass
             # Both vertex stages store their rows in a locality order (rows that gather the same
             # rows of the input follow each other and are processed on one XCD), which cuts
@@ -129,10 +157,15 @@ class CompressGraph():
             # interpreter lock while it runs), so they are computed side by side.
             forward_blocks = (host(self.v2v_graph.csr()), host(self.v2r_graph.csr()))
             backward_blocks = (host(self.v2v_graph.csc()), host(self.r2v_graph.csc()))
+            # From here on the kernels read the plan's own int32 arrays: the int64 blocks go
+            # back to host memory (csr()/csc() still deliver device tensors, as copies), so the
+            # device holds the graph once.  keep_device_blocks = True keeps them resident.
+            if not getattr(self, "keep_device_blocks", False):
+                for block in self.blocks():
+                    block.offload()
             with ThreadPoolExecutor(max_workers=2) as pool:
                 forward_job = pool.submit(ordered, *forward_blocks)
                 backward_job = pool.submit(ordered, *backward_blocks)
-                plan.vertex_stage = stage(*forward_job.result())
-                plan.vertex_stage_t = stage(*backward_job.result())
+                plan.set_vertex_stages(stage(*forward_job.result()), stage(*backward_job.result()))
             self._plan = plan
         return self._plan

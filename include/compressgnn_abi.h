@@ -169,6 +169,14 @@ int cgnn_lsh_scan(int bits, const int32_t *bucket_count, int32_t *prefix, void *
 int cgnn_lsh_finish(int64_t N, int bits, const int32_t *raw_code, const int32_t *bucket_count,
                     const int32_t *prefix, int64_t *ids, int32_t *counts, cgnn_stream_t stream);
 
+/* The bad_id argument of the three entries that read caller-supplied cluster ids
+ * (cgnn_cluster_members, cgnn_cluster_mean_backward, cgnn_reconstruct): a device int32, or
+ * NULL.  The reference traps in the kernel on an id outside [0, groups)
+ * (CUDA_KERNEL_ASSERT, cluster_kernel.cu:74,92); here such an id is treated as the nearest
+ * valid one, so that no access leaves the arrays, and 1 is stored to *bad_id.  0 is never
+ * stored: the caller clears the flag before a call, or a sequence of calls, and reads it
+ * afterwards; the results of a flagged call are meaningless. */
+
 /* Member lists of the clusters: a stable counting sort of the rows by id.
  * offsets[g] = first position of group g in perm (offsets has groups+1 entries),
  * perm[p] = row, sorted_id[p] = its id; rows of one group appear in ascending order.
@@ -176,7 +184,7 @@ int cgnn_lsh_finish(int64_t N, int bits, const int32_t *raw_code, const int32_t 
  * float atomics of sum_features / reconstruct_grad (cluster_kernel.cu:60-69,98-108). */
 size_t cgnn_cluster_members_workspace_bytes(int64_t N, int64_t groups);
 int cgnn_cluster_members(int64_t N, int64_t groups, const int64_t *ids, int32_t *offsets,
-                         int32_t *perm, int32_t *sorted_id, void *workspace,
+                         int32_t *perm, int32_t *sorted_id, int32_t *bad_id, void *workspace,
                          size_t workspace_bytes, cgnn_stream_t stream);
 
 /* Steps 2 and 3 and the member lists in one, from the raw codes alone (no bucket
@@ -209,14 +217,14 @@ int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int64_t max_members,
  * Replaces cluster_mean_backward_cuda (cluster_kernel.cu:171-181). */
 int cgnn_cluster_mean_backward(int64_t N, int64_t F, int64_t groups, int dtype, const void *grad,
                                const int64_t *ids, const int32_t *counts, const int32_t *perm,
-                               void *dx, cgnn_stream_t stream);
+                               void *dx, int32_t *bad_id, cgnn_stream_t stream);
 
 /* out[i,:] = act(reps[ids[i],:] + bias), act(v) = (relu && v < 0) ? 0 : v; bias may be
  * NULL; perm as above (NULL = rows in natural order).
  * Replaces cluster_reconstruct_cuda (cluster_kernel.cu:182-195). */
 int cgnn_reconstruct(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
                      const int64_t *ids, const int32_t *perm, const void *bias, int relu,
-                     void *out, cgnn_stream_t stream);
+                     void *out, int32_t *bad_id, cgnn_stream_t stream);
 
 /* reps_grad[g,:] = sum over members i of g (ascending) of
  * ((relu && output[i,:] <= 0) ? 0 : grad[i,:]).  max_members as for cgnn_cluster_mean.

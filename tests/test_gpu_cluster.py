@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from compressgnn_amd import abi
-from util import assert_within
+from util import assert_no_less_accurate, assert_within
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -204,7 +204,14 @@ def test_large_cluster_sums():
     go = rng.standard_normal((n, F)).astype(np.float32)
     rg = abi.reconstruct_backward(_t(go), _t(out), members, 9, True).cpu().numpy()
     want = oracle.reconstruct_backward(go.astype(np.float64), ids_np, out.astype(np.float64), 9, True)
+    # Sums of up to 18,000 N(0,1) terms (magnitude ~130): two fp32 summation orders differ by
+    # ~1e-4 absolute, beyond the reference test's atol of 1e-5.  The bar that can fail: the
+    # kernel is no further from the float64 sums than the oracle's sequential fp32 scatter-add.
+    sequential = oracle.reconstruct_backward(go, ids_np, out, 9, True)
+    assert_no_less_accurate(rg, sequential, want, factor=1.5)
     np.testing.assert_allclose(rg, want, rtol=1e-4, atol=1e-3)
+    # the means of the same clusters: unnormalised sums are as large, the quotient is small
+    assert_no_less_accurate(reps, oracle.cluster_mean(x, ids_np, counts_np), want64, factor=1.5)
 
 
 def test_memory_probes_move_what_they_say():

@@ -21,33 +21,45 @@ pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
 
 
-def test_propagation_at_full_size():
+@pytest.fixture(scope="module")
+def c1():
+    """The 325,557-vertex copy-model graph of the benchmark, compressed and on the GPU, with the
+    float64 matrix of the uncompressed graph (self loops, symmetric normalisation) beside it."""
+    import scipy.sparse as sp
     import compressgnn_offline as off
     from CompressgnnData import CompressgnnData
-    from KPropagate import KPropagate
-    V, F = 325557, 128
+    V = 325557
     v, e = off.gen_copy_model(V, 9.8, 0.7, 1)
-    rng = np.random.default_rng(12)
-    x_np = rng.standard_normal((V, F)).astype(np.float32)
-    g_np = rng.standard_normal((V, F)).astype(np.float32)
     mask = np.zeros(V, dtype=bool)
-    data = CompressgnnData(x_np, (v, e), np.zeros(V, np.int64), mask, mask, mask, add_self_loop=True,
-                           normalize=True, graph_type="csr", verbose=False)
+    data = CompressgnnData(np.zeros((V, 1), np.float32), (v, e), np.zeros(V, np.int64), mask, mask, mask,
+                           add_self_loop=True, normalize=True, graph_type="csr", verbose=False)
     assert data.rule_cnt > 0
     data.to(DEV)
-    x = data.x.clone().requires_grad_(True)
+    v2, e2 = off.add_self_loop_csr(v, e)
+    d = off.get_norm_degree(e2, V).astype(np.float64)
+    src = np.repeat(np.arange(V), np.diff(v2))
+    A = sp.csr_matrix((d[src] * d[e2], e2, v2), shape=(V, V))  # A[s, d]
+    return data, A
+
+
+@pytest.mark.parametrize("F", [128, 16, 64, 256, 512])
+def test_propagation_at_full_size(c1, F):
+    """The headline width and the widths of the feature sweep, through the layer (the plan:
+    folded rule stage, fused two-source vertex stages in their locality order)."""
+    from KPropagate import KPropagate
+    data, A = c1
+    V = data.vertex_cnt
+    rng = np.random.default_rng(12 + F)
+    x_np = rng.standard_normal((V, F)).astype(np.float32)
+    g_np = rng.standard_normal((V, F)).astype(np.float32)
+    x0 = torch.from_numpy(x_np).to(DEV)
+    x = x0.clone().requires_grad_(True)
     prop = KPropagate()
     out = prop(x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
     g = torch.from_numpy(g_np).to(DEV)
     (gx,) = torch.autograd.grad(out, x, g)
     out_np, gx_np = out.detach().cpu().numpy(), gx.cpu().numpy()
     # forward = A_hat^T x of the uncompressed graph (float64, host), fp32 tolerance of the task
-    v2, e2 = off.add_self_loop_csr(v, e)
-    d = off.get_norm_degree(e2, V).astype(np.float64)
-    src = np.repeat(np.arange(V), np.diff(v2))
-    w = d[src] * d[e2]
-    import scipy.sparse as sp
-    A = sp.csr_matrix((w, e2, v2), shape=(V, V))  # A[s, d]
     want = A.T @ x_np.astype(np.float64)
     assert np.all(np.abs(out_np - want) <= 1e-5 * np.abs(want) + 1e-6)
     # backward = A_hat g, and the adjoint identity ties the two passes together
@@ -57,10 +69,19 @@ def test_propagation_at_full_size():
     rhs = float((x_np.astype(np.float64) * gx_np).sum())
     assert abs(lhs - rhs) <= 1e-6 * max(1.0, abs(lhs))
     # same bits run to run, and linear: P(2x) = 2 P(x) exactly (scaling by two is exact)
-    again = prop(data.x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    again = prop(x0, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
     assert torch.equal(again, out.detach())
-    twice = prop(2 * data.x, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    twice = prop(2 * x0, data.edge_index, None, data.vertex_cnt, data.rule_cnt)
     assert torch.equal(twice, 2 * out.detach())
+    # the forced schedules agree with the chosen one within the same tolerance
+    plan = data.edge_index.plan()
+    try:
+        for method in ("nnz_schedule",) if F > 64 else ("nnz_schedule", "row_schedule"):
+            plan.method = method
+            other = plan.forward(x0).cpu().numpy()
+            assert np.all(np.abs(other - want) <= 1e-5 * np.abs(want) + 1e-6)
+    finally:
+        plan.method = "auto"
 
 
 def test_cluster_path_at_full_size():

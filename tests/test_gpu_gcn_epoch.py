@@ -1,0 +1,145 @@
+"""The large end-to-end configuration at a size a test can check: training epochs of a 2-layer
+GCN whose layers are propagate -> cluster -> Linear on the representatives -> reconstruct(bias)
+(the layer of the reference's model/compressgnn/gcn.py:27-34), ReLU between the layers,
+log-softmax + NLL over all vertices, Adam.  200,000-vertex copy-model graph (the generator and
+average degree of the 18.5 M-vertex benchmark graph), F = hidden = 64, 16 classes, param_H = 16,
+refresh_interval 1 and 5.
+
+Every epoch is compared with a float64 composition of plain torch operators on the same
+parameters: the uncompressed normalised adjacency applied with index_add_, the cluster means
+with index_add_ / counts, the reconstruction with index_select.  The loss and the gradients of
+every parameter and of the input features must agree.  The assignment is not differentiable and
+depends on the last bit of the propagated features, so the composition takes the index tensor
+from the layer; that tensor itself is checked against the oracle's assignment of the features
+the layer hashed (bit-exact)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as Fn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path[:0] = [ROOT, os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compressgnn_amd", "layer"),
+                os.path.join(ROOT, "compressgnn_amd", "loader")]
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+V, AVG_DEGREE, F_IN, HIDDEN, CLASSES, H = 200_000, 16.1, 64, 64, 16, 16
+
+
+@pytest.fixture(scope="module")
+def graph():
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    v, e = off.gen_copy_model(V, AVG_DEGREE, 0.7, 1)
+    mask = np.ones(1, dtype=bool)
+    data = CompressgnnData(np.zeros((V, 1), np.float32), (v, e), np.zeros(1, np.int64), mask, mask, mask,
+                           add_self_loop=True, normalize=True, graph_type="csr", verbose=False)
+    assert data.rule_cnt > 0
+    data.edge_index.to(DEV)
+    # the uncompressed graph as (source, destination, weight) for the torch composition
+    v2, e2 = off.add_self_loop_csr(v, e)
+    d = off.get_norm_degree(e2, V).astype(np.float64)
+    src = np.repeat(np.arange(V), np.diff(v2))
+    edges = (torch.from_numpy(src).to(DEV), torch.from_numpy(e2.astype(np.int64)).to(DEV),
+             torch.from_numpy(d[src] * d[e2]).to(DEV))
+    return data, edges
+
+
+def plain_propagate(edges, x):
+    src, dst, w = edges
+    return torch.zeros_like(x).index_add_(0, dst, w.unsqueeze(1) * x.index_select(0, src))
+
+
+def composition(edges, x, params, indices):
+    """The model in float64 torch operators; params = [(W, b), (W, b)], indices = the two index tensors."""
+    h = x
+    for k, ((W, b), index) in enumerate(zip(params, indices)):
+        h = plain_propagate(edges, h)
+        groups = int(index.max()) + 1
+        counts = torch.bincount(index, minlength=groups).clamp_min(1).to(h.dtype)
+        reps = torch.zeros(groups, h.size(1), dtype=h.dtype, device=h.device).index_add_(0, index, h) / counts[:, None]
+        h = Fn.linear(reps, W, None).index_select(0, index) + b
+        if k == 0:
+            h = h.relu()
+    return Fn.log_softmax(h, dim=1)
+
+
+@pytest.mark.parametrize("refresh_interval", [1, 5])
+def test_gcn_training_epochs_match_a_torch_composition(graph, refresh_interval):
+    from CompressgnnCluster import Compressgnn_Cluster
+    from CompressgnnReconstruct import Compressgnn_Reconstruct
+    from KPropagate import KPropagate
+    data, edges = graph
+    g = data.edge_index
+
+    class Layer(torch.nn.Module):
+        def __init__(self, fin, fout):
+            super().__init__()
+            self.lin = torch.nn.Linear(fin, fout, bias=True)
+            self.P = KPropagate()
+            self.cluster = Compressgnn_Cluster(in_feature=fin, param_H=H, training=True, cache=True,
+                                               refresh_interval=refresh_interval)
+            self.reconstruct = Compressgnn_Reconstruct()
+            self.hashed = None
+
+        def forward(self, x, epoch):
+            x = self.P(x=x, edge_index=g, edge_weight=None, vertex_cnt=data.vertex_cnt, rule_cnt=data.rule_cnt)
+            self.hashed = x.detach()
+            reps, index = self.cluster(x, epoch=epoch)
+            return self.reconstruct(Fn.linear(reps, self.lin.weight, None), index, bias=self.lin.bias)
+
+    torch.manual_seed(refresh_interval)
+    layers = torch.nn.ModuleList([Layer(F_IN, HIDDEN), Layer(HIDDEN, CLASSES)]).to(DEV)
+    opt = torch.optim.Adam(layers.parameters(), lr=0.01)
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    x = torch.randn(V, F_IN, device=DEV, generator=gen).requires_grad_()
+    y = torch.randint(0, CLASSES, (V,), device=DEV, generator=gen)
+    losses, index_ptrs = [], []
+    for epoch in range(7 if refresh_interval > 1 else 3):
+        opt.zero_grad(set_to_none=True)
+        x.grad = None
+        h = layers[0](x, epoch).relu()
+        out = Fn.log_softmax(layers[1](h, epoch), dim=1)
+        loss = -out.gather(1, y.unsqueeze(1)).mean()
+        loss.backward()
+        # the refresh schedule: every `refresh_interval` epochs, the index tensor kept in between
+        for layer in layers:
+            assert layer.cluster.last_refreshed == (epoch % refresh_interval == 0)
+        index_ptrs.append(layers[0].cluster.vertex_index.data_ptr())
+        if epoch % refresh_interval:
+            assert index_ptrs[-1] == index_ptrs[-2]
+        indices = [layer.cluster.vertex_index for layer in layers]
+        if epoch % refresh_interval == 0:
+            # a refreshed assignment is the oracle's assignment of what the layer hashed
+            for layer in layers:
+                want_ids, want_counts, want_active = oracle.assign(layer.hashed.cpu().numpy(),
+                                                                   layer.cluster.random_vectors.cpu().numpy(), H)
+                assert layer.cluster.active_bucket == want_active
+                assert np.array_equal(layer.cluster.vertex_index.cpu().numpy(), want_ids)
+        # the same epoch in float64 torch operators on the same parameters
+        params64 = [(l.lin.weight.detach().double().requires_grad_(), l.lin.bias.detach().double().requires_grad_())
+                    for l in layers]
+        x64 = x.detach().double().requires_grad_()
+        out64 = composition(edges, x64, params64, indices)
+        loss64 = -out64.gather(1, y.unsqueeze(1)).mean()
+        loss64.backward()
+        assert abs(float(loss) - float(loss64)) <= 1e-5 * abs(float(loss64)), (float(loss), float(loss64))
+        assert torch.allclose(out.detach().double(), out64.detach(), rtol=1e-4, atol=1e-5)
+        pairs = [(x.grad, x64.grad)]
+        for layer, (W64, b64) in zip(layers, params64):
+            pairs += [(layer.lin.weight.grad, W64.grad), (layer.lin.bias.grad, b64.grad)]
+        for got, want in pairs:
+            scale = float(want.abs().max())
+            assert scale > 0
+            err = float((got.double() - want).abs().max())
+            assert err <= 2e-5 * scale, (err, scale)
+        losses.append(float(loss))
+        opt.step()
+    assert all(np.isfinite(losses))
+    expected = 3 if refresh_interval == 1 else 2
+    assert [l.cluster.refresh_count for l in layers] == [expected, expected]

@@ -15,7 +15,7 @@ sys.path[:0] = [os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compr
                 os.path.join(ROOT, "compressgnn_amd", "loader")]
 
 import oracle
-from util import assert_within
+from util import assert_no_less_accurate, assert_within
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -74,6 +74,22 @@ def _plain_transpose_product(v, e, x, normalize):
     return out
 
 
+def _plain_product(v, e, g, normalize):
+    """gx = A_hat g of the same graph (the gradient of _plain_transpose_product), in float64."""
+    import compressgnn_offline as off
+    v2, e2 = off.add_self_loop_csr(v, e)
+    V = len(v2) - 1
+    src = np.repeat(np.arange(V), np.diff(v2))
+    if normalize:
+        d = off.get_norm_degree(e2, V).astype(np.float64)
+        w = d[src] * d[e2]
+    else:
+        w = np.ones(len(e2))
+    out = np.zeros((V, g.shape[1]))
+    np.add.at(out, src, w[:, None] * g[e2].astype(np.float64))
+    return out
+
+
 @pytest.mark.parametrize("kind,freq", [("chung_lu", 16), ("chung_lu", 3), ("copy", 3), ("blocks", 16)])
 @pytest.mark.parametrize("normalize", [True, False])
 @pytest.mark.parametrize("F", [128, 16])
@@ -99,9 +115,18 @@ def test_propagate_forward_backward(kind, freq, normalize, F):
     torch.cuda.synchronize()
     want_gx = (oracle.compress_spmm_backward(bwd_blocks, g_np) if data.rule_cnt
                else oracle.spmm(*bwd_blocks["v2v_t"], g_np))
-    tol = dict(rtol=1e-5, atol=1e-6) if normalize else dict(rtol=1e-5, atol=1e-4)
-    assert_within(out.detach().cpu().numpy(), want, **tol)
-    assert_within(gx.cpu().numpy(), want_gx, **tol)
+    if normalize:
+        assert_within(out.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+        assert_within(gx.cpu().numpy(), want_gx, rtol=1e-5, atol=1e-6)
+    else:
+        # unit weights: sums of up to hundreds of O(1) terms, where two summation orders differ
+        # by more than 1e-6 absolute.  The bar that can fail: the kernels are no further from
+        # the float64 product than the oracle's sequential fp32 chain is.
+        plain_g = _plain_product(v, e, g_np, normalize)
+        assert_no_less_accurate(out.detach().cpu().numpy(), want, plain)
+        assert_no_less_accurate(gx.cpu().numpy(), want_gx, plain_g)
+        assert_within(out.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-4)
+        assert_within(gx.cpu().numpy(), want_gx, rtol=1e-5, atol=1e-4)
     # adjoint identity <A x, g> == <x, A^T g> in float64 on the GPU results
     lhs = float((out.detach().cpu().numpy().astype(np.float64) * g_np).sum())
     rhs = float((x_np.astype(np.float64) * gx.cpu().numpy()).sum())
@@ -151,6 +176,9 @@ def test_coo_multi_phase_propagate(kind, freq, normalize):
     tol = dict(rtol=1e-5, atol=1e-6) if normalize else dict(rtol=1e-5, atol=1e-4)
     assert_within(out.detach().cpu().numpy(), want, **tol)
     assert_within(gx.cpu().numpy(), want_gx, **tol)
+    if not normalize:  # the widened bound alone proves little: also no further from float64 than the oracle
+        assert_no_less_accurate(out.detach().cpu().numpy(), want, _plain_transpose_product(v, e, x_np, normalize))
+        assert_no_less_accurate(gx.cpu().numpy(), want_gx, _plain_product(v, e, g_np, normalize))
     assert torch.equal(out, again)
     via_graph = KPropagate()(csr_data.x, csr_data.edge_index, None, csr_data.vertex_cnt, csr_data.rule_cnt)
     assert_within(out.detach().cpu().numpy(), via_graph.cpu().numpy(), **tol)
@@ -162,21 +190,60 @@ def test_coo_multi_phase_propagate(kind, freq, normalize):
 
 
 @pytest.mark.parametrize("fuse", [True, False])
-@pytest.mark.parametrize("method", ["rowbalance", "nnzbalance", "auto"])
+@pytest.mark.parametrize("method", ["row_schedule", "nnz_schedule", "auto", "rowbalance_rowcache"])
 def test_propagate_schedules_agree(fuse, method):
     from CompressgnnSPMM import compress_spmm
     data, _ = _make_data("copy", 64, True, 3)
     fwd_blocks, _ = _np_blocks(data.edge_index)
     want = oracle.compress_spmm_forward(fwd_blocks, data.x.numpy())
     data.to(DEV)
-    data.edge_index.fold_levels = method != "rowbalance"  # one launch per level: the oracle's order of sums
+    data.edge_index.fold_levels = method != "row_schedule"  # one launch per level: the oracle's order of sums
+    data.edge_index.keep_split_blocks = not fuse
     plan = data.edge_index.plan()
+    assert all(b.offloaded for b in data.edge_index.blocks())  # the device holds the plan's arrays only
     plan.fuse_final, plan.method = fuse, method
     out = compress_spmm(data.edge_index, data.x)
     torch.cuda.synchronize()
     assert_within(out.cpu().numpy(), want)
-    if method == "rowbalance":
+    if method == "row_schedule":
         assert np.array_equal(out.cpu().numpy(), want)  # sequential sums in every stage
+
+
+@pytest.mark.parametrize("F", [16, 64, 256, 512])
+@pytest.mark.parametrize("method,fold,fuse", [("auto", True, True), ("nnz_schedule", True, True),
+                                              ("nnz_schedule", False, False), ("row_schedule", False, True),
+                                              ("row_schedule", False, False)])
+def test_plan_feature_sweep(F, method, fold, fuse):
+    """The widths of the feature sweep through the propagation plan itself, forward and
+    gradient: folded rule stage and fused two-source vertex stages (F = 512 takes two feature
+    tiles per lane), both schedules, and the launch-per-level / two-launch forms, against the
+    oracle's 4-stage chain at 1e-5 relative / 1e-6 absolute.  A forced row schedule with one
+    launch per level sums in the oracle's order: same bits."""
+    data, _ = _make_data("copy", F, True, 3, seed=F)
+    graph = data.edge_index
+    assert data.rule_cnt > 0 and graph.step >= 1
+    fwd_blocks, bwd_blocks = _np_blocks(graph)
+    x_np = data.x.numpy().copy()
+    g_np = np.random.default_rng(F).standard_normal(x_np.shape).astype(np.float32)
+    want = oracle.compress_spmm_forward(fwd_blocks, x_np)
+    want_g = oracle.compress_spmm_backward(bwd_blocks, g_np)
+    data.to(DEV)
+    graph.fold_levels, graph.keep_split_blocks = fold, not fuse
+    plan = graph.plan()
+    assert graph.levels_folded == fold
+    plan.fuse_final, plan.method = fuse, method
+    out = plan.forward(data.x)
+    gx = plan.backward(torch.from_numpy(g_np).to(DEV))
+    torch.cuda.synchronize()
+    assert_within(out.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+    assert_within(gx.cpu().numpy(), want_g, rtol=1e-5, atol=1e-6)
+    if method == "row_schedule":
+        assert np.array_equal(out.cpu().numpy(), want) and np.array_equal(gx.cpu().numpy(), want_g)
+    if not fuse:
+        with pytest.raises(RuntimeError):  # a plan built without the split blocks says so
+            other, _ = _make_data("copy", 16, True, 3, seed=F)
+            other.to(DEV)
+            other.edge_index.plan().fuse_final = False
 
 
 def test_propagation_replays_from_a_captured_graph():
@@ -324,3 +391,169 @@ def test_cluster_reconstruct_layers():
                                atol=1e-5, rtol=1e-4)
     with pytest.raises(RuntimeError):
         native.cluster_assign(x, torch.randn(7, 3, device=DEV), 4, native.cluster_workspace(x, 4))
+
+
+def test_kpu_propagate_hops_and_cache():
+    """KPUPropagate (layer/KPUPropagate.py:25-37 of the reference): K hops per call; with
+    cached=True the first result is kept and later calls return it detached, whatever their
+    arguments, until reset_cache()."""
+    from KPropagate import KPropagate
+    from KPUPropagate import KPUPropagate
+    data, _ = _make_data("copy", 32, True, 3, seed=2)
+    data.to(DEV)
+    args = (data.edge_index, None, data.vertex_cnt, data.rule_cnt)
+    x = data.x.detach().clone().requires_grad_()
+    hop = KPropagate()
+    two = hop(hop(x, *args), *args)
+    g = torch.randn(two.shape, device=DEV, generator=torch.Generator(device=DEV).manual_seed(1))
+    (gx_two,) = torch.autograd.grad(two, x, g)
+    kpu = KPUPropagate(K=2)
+    out = kpu(x, *args)
+    (gx,) = torch.autograd.grad(out, x, g)
+    assert torch.equal(out, two) and torch.equal(gx, gx_two)  # the same kernels in the same order
+    assert out.requires_grad and "K=2" in repr(kpu)
+    # one hop of K=1 is KPropagate, and K=3 is one more hop on top of K=2
+    assert torch.equal(KPUPropagate(K=1)(x, *args), hop(x, *args))
+    assert torch.equal(KPUPropagate(K=3)(x, *args), hop(two, *args))
+    # against the oracle: two applications of the compressed chain
+    fwd_blocks, _ = _np_blocks(data.edge_index)
+    want = oracle.compress_spmm_forward(fwd_blocks, oracle.compress_spmm_forward(fwd_blocks, data.x.cpu().numpy()))
+    assert_within(out.detach().cpu().numpy(), want)
+
+    cached = KPUPropagate(K=2, cached=True)
+    first = cached(x, *args)
+    assert first.requires_grad and torch.equal(first, two)
+    other = torch.randn_like(x)
+    second = cached(other, *args)  # arguments are ignored while the cache is filled
+    assert not second.requires_grad and second.data_ptr() == first.data_ptr() and torch.equal(second, two)
+    third = cached(other, *args)
+    assert third.data_ptr() == first.data_ptr() and not third.requires_grad
+    cached.reset_cache()
+    fresh = cached(other, *args)
+    assert fresh.data_ptr() != first.data_ptr()
+    assert torch.equal(fresh, hop(hop(other, *args), *args))
+    # without the cache every call propagates its own input
+    plain = KPUPropagate(K=2, cached=False)
+    assert torch.equal(plain(other, *args), fresh) and torch.equal(plain(x, *args), two)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,width,bits", [(1, 5, 0), (67, 33, 8), (5000, 100, 12), (257, 128, 16), (300, 7, 20)])
+def test_cluster_forward_entry(dtype, n, width, bits):
+    """compressgnn_runtime.cluster_forward (src/runtime/csrc/cluster/cluster.cpp:12-30 of the
+    reference): int32 ids, 1-based and dense in code order, and the number of active buckets."""
+    import compressgnn_runtime as rt
+    rng = np.random.default_rng(31 * n + bits)
+    x = rng.standard_normal((n, width)).astype(dtype)
+    planes = rng.standard_normal((width, bits)).astype(dtype)
+    want_ids, want_active, _ = oracle.lsh(x, planes, bits)
+    ids, active = rt.cluster_forward(torch.from_numpy(x).to(DEV), torch.from_numpy(planes).to(DEV), bits)
+    assert ids.dtype == torch.int32 and ids.shape == (n,) and ids.is_cuda
+    assert active == want_active
+    assert np.array_equal(ids.cpu().numpy(), np.asarray(want_ids).astype(np.int32))
+    with pytest.raises(RuntimeError):
+        rt.cluster_forward(torch.from_numpy(x).to(DEV), torch.from_numpy(planes).to(DEV), bits + 1)
+    with pytest.raises(RuntimeError):
+        rt.cluster_forward(torch.from_numpy(x), torch.from_numpy(planes), bits)  # CPU tensors
+
+
+def test_cluster_operators_reject_bad_operands():
+    """Every operand check raises RuntimeError (the reference's TORCH_CHECKs do); ids that name
+    no cluster are reported instead of read (the reference traps in the kernel)."""
+    import compressgnn_runtime as rt
+    x = torch.randn(50, 8, device=DEV)
+    planes = torch.randn(8, 4, device=DEV)
+    ids, counts, active = rt.cluster_assign(x, planes, 4, rt.cluster_workspace(x, 4))
+    groups = active + 1
+    reps = rt.cluster_mean(x, ids, counts)
+    bad_calls = [
+        lambda: rt.cluster_workspace(x, 31),
+        lambda: rt.cluster_workspace(x.to(torch.int32), 4),
+        lambda: rt.cluster_assign(x, planes, 4, rt.cluster_workspace(x, 5)),       # workspace of another size
+        lambda: rt.cluster_assign(x, planes, 4, rt.cluster_workspace(x, 4)[:2]),
+        lambda: rt.cluster_assign(x, planes.double(), 4, rt.cluster_workspace(x, 4)),
+        lambda: rt.cluster_assign(x.t(), planes, 4, rt.cluster_workspace(x, 4)),  # not contiguous
+        lambda: rt.cluster_mean(x, ids.to(torch.int32), counts),
+        lambda: rt.cluster_mean(x, ids[:-1], counts),
+        lambda: rt.cluster_mean(x, ids, counts.to(torch.int64)),
+        lambda: rt.cluster_mean(x, ids.cpu(), counts),
+        lambda: rt.cluster_mean_backward(reps[:-1], ids, counts),
+        lambda: rt.cluster_reconstruct(reps, ids, torch.zeros(7, device=DEV), False),
+        lambda: rt.cluster_reconstruct(reps, ids, torch.zeros(8, device=DEV, dtype=torch.double), False),
+        lambda: rt.cluster_reconstruct_backward(torch.zeros(50, 8, device=DEV), ids, torch.zeros(50, 9, device=DEV),
+                                                groups, True),
+        lambda: rt.cluster_members(ids, 0),
+    ]
+    for k, call in enumerate(bad_calls):
+        with pytest.raises(RuntimeError):
+            call()
+            raise AssertionError("bad call %d was accepted" % k)
+    # ids beyond the representatives: an error, never an access outside the arrays
+    beyond = ids.clone()
+    beyond[7] = groups + 3
+    negative = ids.clone()
+    negative[0] = -1
+    for index in (beyond, negative):
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_reconstruct(reps, index, None, False)
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_mean_backward(reps, index, counts)
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_members(index, groups)
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_mean(x, index, counts)  # builds the member lists itself
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_reconstruct_backward(torch.zeros(50, 8, device=DEV), index, torch.ones(50, 8, device=DEV),
+                                            groups, True)
+    # the device is fine afterwards and the good calls still give the same results
+    torch.cuda.synchronize()
+    assert torch.equal(rt.cluster_mean(x, ids, counts), reps)
+    from CompressgnnReconstruct import Compressgnn_Reconstruct
+    with pytest.raises(RuntimeError, match="outside"):
+        Compressgnn_Reconstruct()(reps, beyond)
+
+
+def test_reference_method_strings_are_hints():
+    """The reference's layers ask for "rowbalance_rowcache" on every block of 1e6 non-zeros and
+    width >= 64 (layer/CompressgnnSPMM.py:14-19,34,38), whatever its rows look like.  On a block
+    with power-law rows the string must not force a lane group per row: same result as "auto"
+    (bit for bit: the same schedule runs), within tolerance of the oracle, and no slower than a
+    small multiple of "auto"."""
+    import compressgnn_runtime as rt
+    rng = np.random.default_rng(8)
+    rows, cols, F = 60000, 60000, 64
+    lens = np.minimum((rng.pareto(1.1, rows) * 3).astype(np.int64) + 1, 40000)
+    lens[rng.integers(0, rows, 3)] = 60000  # three hub rows
+    vlist = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    elist = rng.integers(0, cols, int(vlist[-1])).astype(np.int64)
+    value = (rng.standard_normal(len(elist)) * 0.3 / np.sqrt(np.repeat(lens, lens))).astype(np.float32)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    tv, te, tw, tx = t(vlist), t(elist), t(value), t(x)
+    auto = rt.spmm_func(tv, te, tw, tx, "auto", None)
+    hinted = rt.spmm_func(tv, te, tw, tx, "rowbalance_rowcache", None)
+    assert torch.equal(auto, hinted)
+    want = oracle.spmm(vlist, elist, value, x, None, 8)
+    # rows of up to 60,000 entries: the sequential fp32 sum is itself several 1e-6 from the exact
+    # value, so the kernel is held to being no further from float64 than the oracle is
+    truth = np.zeros((rows, F))
+    np.add.at(truth, np.repeat(np.arange(rows), lens), value[:, None].astype(np.float64) * x[elist])
+    assert_no_less_accurate(hinted.cpu().numpy(), want, truth, factor=1.5)
+    assert_within(hinted.cpu().numpy(), want, rtol=1e-4, atol=1e-5)
+
+    def timed(method):
+        rt.spmm_func(tv, te, tw, tx, method, None)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            rt.spmm_func(tv, te, tw, tx, method, None)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / 5
+
+    t_auto, t_hint = timed("auto"), timed("rowbalance_rowcache")
+    assert t_hint <= 1.5 * t_auto + 0.05, (t_hint, t_auto)
+    # a forced row schedule stays available under this build's own name, bit-exact with the oracle
+    forced = rt.DeviceCsr(tv, te, tw, rows, cols, torch.device(DEV)).spmm(tx, None, "row_schedule")
+    assert np.array_equal(forced.cpu().numpy(), want)

@@ -179,3 +179,94 @@ def test_a_prepared_dataset_survives_torch_save(tmp_path):
             assert torch.equal(a, b)
     assert again.edge_index.step == data.edge_index.step
     assert torch.equal(again.edge_index.vertex_degree, data.edge_index.vertex_degree)
+
+
+def _binary_hierarchy(depth, width=2):
+    """A compressed graph whose rules form `depth` levels of `width` rules each; every rule
+    above the lowest level has all rules of the level below as children, so the vertices a
+    rule stands for multiply by `width` per level while the stored entries grow by width^2."""
+    V = 2 * width + 1
+    rules = depth * width
+    rows = [[] for _ in range(V + rules)]
+    rid = lambda level, k: V + level * width + k
+    for k in range(width):
+        rows[rid(0, k)] = [1 + 2 * k, 2 + 2 * k]
+    for level in range(1, depth):
+        for k in range(width):
+            rows[rid(level, k)] = [rid(level - 1, j) for j in range(width)]
+    rows[0] = [rid(depth - 1, k) for k in range(width)]  # vertex 0 points at the top rules
+    for v in range(1, V):
+        rows[v] = [0]
+    vlist = np.concatenate([[0], np.cumsum([len(r) for r in rows])]).astype(np.int64)
+    elist = np.array([c for r in rows for c in r], dtype=np.int64)
+    weight = np.ones(len(elist), np.float32)
+    colptr, row, value = off.csr_transpose(vlist, elist, weight, V + rules)
+    return CompressGraph(colptr, row, value, V), V, rules
+
+
+def test_fold_bound_and_fallback_for_deep_hierarchies():
+    """plan() folds the rule levels into the rule stage only while that stays cheap: the
+    size bound (row lengths only) is exact when no columns merge and an upper bound otherwise,
+    and a hierarchy whose folded rows would multiply out, or that is deeper than the limit,
+    keeps one launch per level."""
+    host = lambda triple: tuple(t.cpu().numpy() for t in triple)
+    # a shallow hierarchy folds
+    shallow, V, R = _binary_hierarchy(3)
+    assert shallow.step == 2 and shallow.rule_cnt == R
+    folded = shallow._fold_plan(host)
+    assert folded is not None
+    for base, levels, widest in ((folded[0], folded[1], 1), (folded[2], folded[3], 4)):
+        bound = off.csr_fold_levels_bound(base, levels)
+        rp, ci, val = off.csr_fold_levels(base, levels)
+        assert bound >= len(ci) and bound <= 4.0 * (len(base[1]) + sum(len(l[1]) for l in levels))
+        # forward, every rule descends from vertex 0 alone; backward, a top rule stands for the
+        # four vertices below the lowest rules (reached along several paths, merged by column)
+        assert np.diff(rp).max() == widest
+    # exponential growth: 14 levels of 2 rules would fold into rows of 2^14 entries before merging
+    deep, V, R = _binary_hierarchy(14)
+    assert deep.step == 13
+    fwd_base, fwd_levels = host(deep.r2v_graph.csr()), [host(g.csr()) for g in deep.r2r_graph]
+    stored = len(fwd_base[1]) + sum(len(l[1]) for l in fwd_levels)
+    assert off.csr_fold_levels_bound(fwd_base, fwd_levels) > 4.0 * stored
+    assert deep._fold_plan(host) is None
+    # a chain deeper than max_fold_depth is not folded even though it would not grow
+    chain, V, R = _binary_hierarchy(20, width=1)
+    assert chain.step == 19 and chain.step > CompressGraph.max_fold_depth
+    assert chain._fold_plan(host) is None
+    chain.max_fold_depth = 32
+    assert chain._fold_plan(host) is not None
+    # fold_levels = False always keeps the launch-per-level form
+    shallow.fold_levels = False
+    assert shallow._fold_plan(host) is None
+    # random levels: the bound is never below the folded size
+    rng = np.random.default_rng(3)
+    Rn, Vn = 50, 30
+
+    def to_csr(m):
+        rp = np.concatenate([[0], np.cumsum((m != 0).sum(1))]).astype(np.int64)
+        rows, cols = np.nonzero(m)
+        return rp, cols.astype(np.int64), m[rows, cols].astype(np.float32)
+
+    dense = np.where(rng.random((Rn, Vn)) < 0.2, 1.0, 0.0).astype(np.float32)
+    lv = []
+    for k in range(2):
+        L = np.zeros((Rn, Rn), np.float32)
+        lo, hi = 10 * k + 10, 10 * k + 20
+        L[lo:hi, :lo] = rng.random((hi - lo, lo)) < 0.3
+        lv.append(to_csr(L))
+    rp, ci, _ = off.csr_fold_levels(to_csr(dense), lv)
+    assert off.csr_fold_levels_bound(to_csr(dense), lv) >= len(ci)
+
+
+def test_offloaded_blocks_deliver_to_their_device():
+    """SparseCSR.offload(): the arrays rest on the host, the block still answers for its
+    device (here the host itself, which makes offload a no-op that must change nothing)."""
+    data, v, e = make("copy")
+    g = data.edge_index.v2v_graph
+    before = tuple(t.clone() for t in g.csr())
+    csc_before = tuple(t.clone() for t in g.csc())
+    assert not g.offloaded
+    g.offload()
+    assert not g.offloaded and g.device.type == "cpu"
+    assert all(torch.equal(a, b) for a, b in zip(g.csr(), before))
+    assert all(torch.equal(a, b) for a, b in zip(g.csc(), csc_before))
