@@ -128,7 +128,8 @@ def test_gcn_training_epochs_match_a_torch_composition(graph, refresh_interval):
         out64 = composition(edges, x64, params64, indices)
         loss64 = -out64.gather(1, y.unsqueeze(1)).mean()
         loss64.backward()
-        assert abs(float(loss) - float(loss64)) <= 1e-5 * abs(float(loss64)), (float(loss), float(loss64))
+        loss_f, loss64_f = float(loss.detach()), float(loss64.detach())
+        assert abs(loss_f - loss64_f) <= 1e-5 * abs(loss64_f), (loss_f, loss64_f)
         assert torch.allclose(out.detach().double(), out64.detach(), rtol=1e-4, atol=1e-5)
         pairs = [(x.grad, x64.grad)]
         for layer, (W64, b64) in zip(layers, params64):
@@ -138,7 +139,7 @@ def test_gcn_training_epochs_match_a_torch_composition(graph, refresh_interval):
             assert scale > 0
             err = float((got.double() - want).abs().max())
             assert err <= 2e-5 * scale, (err, scale)
-        losses.append(float(loss))
+        losses.append(loss_f)
         opt.step()
     assert all(np.isfinite(losses))
     expected = 3 if refresh_interval == 1 else 2
