@@ -18,6 +18,7 @@ SPMM_AUTO, SPMM_ROW, SPMM_NNZ = 0, 1, 2
 EXPORTS = [
     "cgnn_last_error", "cgnn_version",
     "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
+    "cgnn_spmm_static_scratch_bytes", "cgnn_spmm_static",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
     "cgnn_csr_transpose_workspace_bytes", "cgnn_csr_transpose_device",
     "cgnn_compress_batch_workspace_bytes", "cgnn_compress_csr_batch_device",
@@ -50,7 +51,7 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.cgnn_last_error.restype = ctypes.c_char_p
         L.cgnn_version.restype = ctypes.c_char_p
-        for name in ("cgnn_spmm_workspace_bytes", "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_group_workspace_bytes",
+        for name in ("cgnn_spmm_workspace_bytes", "cgnn_spmm_static_scratch_bytes", "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_group_workspace_bytes",
                      "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes",
                      "cgnn_csr_transpose_workspace_bytes", "cgnn_compress_batch_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
@@ -149,6 +150,15 @@ def spmm(A, X, Y=None, accumulate=False, kernel=SPMM_AUTO):
     check(lib().cgnn_spmm(ctypes.byref(s), dtype_code(X.dtype), ptr(X), ptr(Y), i64(F),
                           ctypes.c_int(1 if accumulate else 0), ctypes.c_int(kernel), ptr(ws),
                           ctypes.c_size_t(need), stream_of(X)))
+    return Y
+
+
+def spmm_static(A, X, Y, accumulate=False, kernel=SPMM_AUTO):
+    """Y (+)= A @ X through cgnn_spmm_static: the caller brings X and Y, the library its own
+    scratch; nothing is allocated by the call."""
+    s = A.struct()
+    check(lib().cgnn_spmm_static(ctypes.byref(s), dtype_code(X.dtype), ptr(X), ptr(Y), i64(X.shape[1]),
+                                 ctypes.c_int(1 if accumulate else 0), ctypes.c_int(kernel), stream_of(X)))
     return Y
 
 

@@ -39,6 +39,7 @@
 // X may alias Y when accumulating (rule levels are updated in place, reference
 // layer/CompressgnnSPMM.py:56-58), so X and Y carry no __restrict__; a row that is
 // written is never gathered in the same launch (levels only read earlier levels).
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -1095,9 +1096,76 @@ int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, voi
     return fail(CGNN_EUNSUPPORTED, "spmm: dtype must be f32 or f64");
 }
 
+// ------------------------------------------- scratch that nobody allocates -------
+//
+// cgnn_spmm_static runs the same kernels as cgnn_spmm with the carries of the nnz schedule in
+// an array that is part of the library's device image, for callers that cannot allocate.
+// Every GPU the library runs on holds its own copy of the array, at its own address, from the
+// moment the image is loaded there until the process ends.
+constexpr size_t kStaticScratchBytes = size_t(64) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex static_scratch_lock;
+void *static_scratch_of_device[kMaxDevices] = {};
+
+// The address of `scratch` on the device that is current in the calling thread.  In host code
+// the name `scratch` is only a handle for the symbol: the device address comes from
+// hipGetSymbolAddress, once per device, and is what kernels and copies are given.
+int static_scratch(void **out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+        set_error("cgnn_spmm_static: no usable current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return CGNN_ELAUNCH;
+    }
+    std::lock_guard<std::mutex> hold(static_scratch_lock);
+    if (static_scratch_of_device[device] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            set_error("cgnn_spmm_static: hipGetSymbolAddress failed on device %d: %s", device, hipGetErrorString(e));
+            return CGNN_ELAUNCH;
+        }
+        static_scratch_of_device[device] = ptr;
+    }
+    *out = static_scratch_of_device[device];
+    return CGNN_OK;
+}
+
+}  // namespace
+
 }  // namespace cgnn
 
 using namespace cgnn;
+
+extern "C" size_t cgnn_spmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int cgnn_spmm_static(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F, int accumulate,
+                                int kernel, cgnn_stream_t stream) {
+    int rc = check_csr(A, "cgnn_spmm_static");
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(F >= 0, "cgnn_spmm_static: F must be non-negative");
+    CGNN_REQUIRE(kernel >= CGNN_SPMM_AUTO && kernel <= CGNN_SPMM_NNZ, "cgnn_spmm_static: unknown kernel id");
+    CGNN_REQUIRE(dtype == CGNN_F32 || dtype == CGNN_F64, "cgnn_spmm_static: dtype must be f32 or f64");
+    const size_t need = cgnn_spmm_workspace_bytes(A, F, dtype, kernel);
+    if (need > kStaticScratchBytes) {
+        set_error("cgnn_spmm_static: this product needs %zu bytes of scratch, the built-in array holds %zu; use "
+                  "cgnn_spmm with a workspace of the caller's",
+                  need, kStaticScratchBytes);
+        return CGNN_EWORKSPACE;
+    }
+    void *ws = nullptr;
+    if (need > 0) {
+        rc = static_scratch(&ws);
+        if (rc != CGNN_OK) return rc;
+    }
+    // The kernels write every carry slot and every carry-row entry they later read, so the
+    // contents a previous call left in the array need no clearing.
+    return cgnn_spmm(A, dtype, X, Y, F, accumulate, kernel, ws, need > 0 ? kStaticScratchBytes : 0, stream);
+}
 
 extern "C" size_t cgnn_spmm_workspace_bytes(const cgnn_csr *A, int64_t F, int dtype, int kernel) {
     if (A == nullptr || A->nnz <= 0 || F <= 0) return 0;

@@ -88,6 +88,21 @@ int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
               int accumulate, int kernel, void *workspace, size_t workspace_bytes,
               cgnn_stream_t stream);
 
+/* cgnn_spmm with the scratch of the nnz schedule inside the library: no workspace argument, and
+ * the call allocates nothing (no hipMalloc, no hipFree, no allocating library routine).  It has
+ * no counterpart in the reference; it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation.  X, Y and the block are the
+ * caller's as in cgnn_spmm, and the result is the same bit for bit.  The scratch is one array of
+ * cgnn_spmm_static_scratch_bytes() bytes (64 MiB) in the library's device image; each GPU the
+ * library runs on holds its copy until the process ends.  A product whose
+ * cgnn_spmm_workspace_bytes exceeds that is refused with CGNN_EWORKSPACE (at F = 128 and the
+ * default run length that is about 8 M non-zeros in the nnz schedule; the row schedule needs no
+ * scratch and has no limit).  All calls on one GPU share the one array: calls that overlap
+ * in time on the same GPU (two streams, two threads) race on it. */
+size_t cgnn_spmm_static_scratch_bytes(void);
+int cgnn_spmm_static(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
+                     int accumulate, int kernel, cgnn_stream_t stream);
+
 /* Two-source product in one pass: A has `cols` columns; a column c < split gathers
  * row c of X0, a column c >= split gathers row c - split of X1.  Every row of Y is
  * written as (0 + S1) + S0 with S1 / S0 the sums over the row's X1 / X0 entries, each
