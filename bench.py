@@ -13,11 +13,12 @@ resident in HBM.  Prints ONE JSON line:
                HIP events inside the timed region
   cpu_baseline the same step on the host cores (the reference's own CPU operator when
                oracle/_ref is built, else the C oracle), timed in this run
-  detail       per-stage times, plain-CSR comparison, cluster + reconstruct times (C3)
+  detail       per-stage times, plain-CSR comparison, the feature sweep F in {16, 64, 256, 512}
+               (C2), cluster + reconstruct times (C3), the 2-layer GCN epoch on the 18.5 M-vertex
+               graph (C4: epoch ms and peak HBM)
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cluster] [--skip-cpu]
-       python bench.py --c4 [--c4-vertices N]   (the large end-to-end configuration only:
-                                                 minutes of host-side graph preparation)
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cluster] [--skip-cpu] [--skip-sweep] [--skip-c4]
+       python bench.py --c4 [--c4-vertices N]   (the large end-to-end configuration only)
 """
 import argparse
 import json
@@ -42,17 +43,33 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def git_blob_hash(path):
+    """The hash `git hash-object` gives the file: names the exact source a figure was measured on."""
+    import hashlib
+    data = open(path, "rb").read()
+    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+
+
 def recorded_traffic():
-    """HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc runs
-    summarised in profiles/ (FETCH_SIZE and WRITE_SIZE scaled by the copy-kernel probe)."""
+    """HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc runs summarised in
+    profiles/ (FETCH_SIZE and WRITE_SIZE scaled by the copy-kernel probe).  The summary names the
+    git blob of csrc/spmm.hip it was measured on; (bytes, note): the note is None when that is
+    the kernel source of this run and says so when the source has changed since."""
     path = os.path.join(ROOT, "profiles", "spmm_nnz_dual_C1_F128_pmc.txt")
+    traffic, measured_on = None, None
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch"):
-                return int(float(line.split("=")[1]))
+                traffic = int(float(line.split("=")[1]))
+            if line.startswith("spmm_hip_blob"):
+                measured_on = line.split("=")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, "profiles/spmm_nnz_dual_C1_F128_pmc.txt not found"
+    current = git_blob_hash(os.path.join(PKG, "csrc", "spmm.hip"))
+    if measured_on != current:
+        return traffic, ("STALE: counters were collected on csrc/spmm.hip blob %s, this run's source is blob %s"
+                         % (measured_on, current))
+    return traffic, None
 
 
 def block_bytes(rowptr, col, ncols, F, acc, elt=4):
@@ -398,7 +415,13 @@ def main():
     ap.add_argument("--features", type=int, default=128)
     ap.add_argument("--skip-cluster", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--sweep", action="store_true", help="also time F in {16, 64, 256, 512} (C2)")
+    ap.add_argument("--skip-sweep", action="store_true", help="leave out the feature sweep F in {16, 64, 256, 512} (C2)")
+    ap.add_argument("--skip-c4", action="store_true",
+                    help="leave out the large end-to-end leg (C4: about two minutes of graph preparation)")
+    ap.add_argument("--windowed-probe", action="store_true",
+                    help="also time the kernels on a graph with the row lengths of C1 whose gathers stay in L2")
+    ap.add_argument("--stream-rows-over", type=int, default=0,
+                    help="forward vertex stage: streaming loads for the runs of rows longer than this (0 = off)")
     ap.add_argument("--c4", action="store_true",
                     help="run only the large end-to-end configuration (2-layer GCN epoch) and print its line")
     ap.add_argument("--c4-vertices", type=int, default=C4_VERTICES)
@@ -424,6 +447,7 @@ def main():
     acct = graph_accounting(graph, F)
     data.to(dev)
     plan = graph.plan()
+    plan.vertex_stage.stream_rows_over = args.stream_rows_over
     gen = torch.Generator(device=dev)
     gen.manual_seed(7)
     x = torch.randn(C1_VERTICES, F, device=dev, generator=gen)
@@ -444,6 +468,9 @@ def main():
     stages = stage_means(plan.take_stage_times())
     plan.timed_stages = []
 
+    workload = {"workload": "C1: copy-model web graph, 325,557 vertices / %d directed edges (+ self loops, "
+                            "sym-norm), compressed propagation forward + backward, F=%d fp32" % (len(e_raw), F),
+                "rules": int(data.rule_cnt), "levels": int(graph.step)}
     step_bytes = sum(a["bytes"] for a in acct.values())
     step_flops = sum(a["flops"] for a in acct.values())
     value = step_bytes / (ms_step * 1e-3) / 1e9
@@ -480,36 +507,37 @@ def main():
                                              forward_GBps=pb_f["bytes"] / (f_ms * 1e-3) / 1e9,
                                              backward_GBps=pb_b["bytes"] / (b_ms * 1e-3) / 1e9,
                                              forward_bytes=pb_f["bytes"], backward_bytes=pb_b["bytes"])
-    # the same kernels on a graph whose gathers stay in L2: row lengths and weights of the C1 graph,
-    # neighbours drawn from a window of 2,048 vertices around the row instead of the copy model
-    rng_l = np.random.default_rng(11)
-    src_l = np.repeat(np.arange(C1_VERTICES, dtype=np.int64), np.diff(v2))
-    col_l = (src_l + rng_l.integers(-1024, 1024, size=len(src_l))) % C1_VERTICES
-    col_l = col_l[np.argsort(src_l * C1_VERTICES + col_l, kind="stable")]
-    local = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(col_l), torch.from_numpy(w), C1_VERTICES,
-                         C1_VERTICES, dev)
-    lb = block_bytes(v2, col_l, C1_VERTICES, F, 0)
-    detail["windowed_graph_same_row_lengths"] = {}
-    for name, forced in (("rowbalance", "row_schedule"), ("nnzbalance", "nnz_schedule")):
-        l_ms = time_loop(lambda: local.spmm(x, None, forced), args.steps, 2, torch)
-        detail["windowed_graph_same_row_lengths"][name] = dict(ms=l_ms, bytes=lb["bytes"],
-                                                               GBps=lb["bytes"] / (l_ms * 1e-3) / 1e9)
-    del local
+    if args.windowed_probe:
+        # the same kernels on a graph whose gathers stay in L2: row lengths and weights of the C1 graph,
+        # neighbours drawn from a window of 2,048 vertices around the row instead of the copy model
+        rng_l = np.random.default_rng(11)
+        src_l = np.repeat(np.arange(C1_VERTICES, dtype=np.int64), np.diff(v2))
+        col_l = (src_l + rng_l.integers(-1024, 1024, size=len(src_l))) % C1_VERTICES
+        col_l = col_l[np.argsort(src_l * C1_VERTICES + col_l, kind="stable")]
+        local = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(col_l), torch.from_numpy(w), C1_VERTICES,
+                             C1_VERTICES, dev)
+        lb = block_bytes(v2, col_l, C1_VERTICES, F, 0)
+        detail["windowed_graph_same_row_lengths"] = {}
+        for name, forced in (("rowbalance", "row_schedule"), ("nnzbalance", "nnz_schedule")):
+            l_ms = time_loop(lambda: local.spmm(x, None, forced), args.steps, 2, torch)
+            detail["windowed_graph_same_row_lengths"][name] = dict(ms=l_ms, bytes=lb["bytes"],
+                                                                   GBps=lb["bytes"] / (l_ms * 1e-3) / 1e9)
+        del local
     # parity of the measured configuration: compressed == plain within tolerance
     out, gx = step()
     ref_out = plain_t.spmm(x, None, "row_schedule")
     err = (out - ref_out).abs().max().item()
     detail["max_abs_diff_vs_plain_csr"] = err
 
-    if args.sweep:
+    if not args.skip_sweep:
         sweep = {}
         for Fs in (16, 64, 256, 512):
             xs = torch.randn(C1_VERTICES, Fs, device=dev, generator=gen)
             gs = torch.randn(C1_VERTICES, Fs, device=dev, generator=gen)
             ms = time_loop(lambda: (plan.forward(xs), plan.backward(gs)), args.steps, 2, torch)
-            a = graph_accounting(graph.to("cpu") if False else graph, Fs)
-            nbytes = sum(t["bytes"] for t in a.values())
-            sweep[str(Fs)] = dict(ms_per_step=ms, bytes=nbytes, GBps=nbytes / (ms * 1e-3) / 1e9)
+            nbytes = sum(t["bytes"] for t in graph_accounting(graph, Fs).values())
+            sweep[str(Fs)] = dict(ms_per_step=ms, bytes=nbytes, GBps=nbytes / (ms * 1e-3) / 1e9,
+                                  frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS)
             del xs, gs
         detail["feature_sweep_C2"] = sweep
 
@@ -545,18 +573,32 @@ def main():
         if not args.skip_cpu:
             cpu_cluster_baseline(xc, planes, detail)
 
+    if not args.skip_c4:
+        # the large end-to-end configuration, after everything of C1 and C3 has left the device
+        del x, g, out, gx, ref_out, plan, graph, data
+        xc = planes = None
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        try:
+            c4 = bench_c4(torch, args.c4_vertices, args.c4_epochs, args.c4_refresh_interval)
+            detail["gcn_epoch_C4"] = dict(ms_per_epoch=c4["value"], workload=c4["config"]["workload"],
+                                          rules=c4["config"]["rules"], levels=c4["config"]["levels"], **c4["detail"])
+        except Exception as exc:  # the headline line must not depend on this leg
+            detail["gcn_epoch_C4"] = dict(error="%s: %s" % (type(exc).__name__, exc))
+            log("[bench] C4 leg failed: %r" % (exc,))
+
+    traffic, traffic_note = recorded_traffic()
     result = {
         "metric": "compressed_propagate_fwd_bwd_hbm_GBps_F%d" % F,
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "C1: copy-model web graph, 325,557 vertices / %d directed edges (+ self loops, "
-                               "sym-norm), compressed propagation forward + backward, F=%d fp32" % (len(e_raw), F),
-                   "rules": int(data.rule_cnt), "levels": int(graph.step)},
+        "config": workload,
         "frac_of_hbm_peak": value / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "cgnn_spmm_dual, forward vertex stage [v2v | v2r]: spmm_nnz_kernel<float,4,32,1,dual> + its fix-up pass",
                      "achieved": dom_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom_gbps / HBM_PEAK_GBPS,
-                     "traffic": recorded_traffic(), "ms": dom, "bytes": dom_bytes},
+                     "traffic": traffic, "traffic_note": traffic_note, "ms": dom, "bytes": dom_bytes},
         "cpu_baseline": cpu,
         "detail": detail,
     }

@@ -35,7 +35,7 @@ class CsrStruct(ctypes.Structure):
         ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("nnz", ctypes.c_int64),
         ("rowptr", ctypes.c_void_p), ("colidx", ctypes.c_void_p), ("rowidx", ctypes.c_void_p),
         ("val", ctypes.c_void_p), ("max_row_nnz", ctypes.c_int32), ("seg_nnz", ctypes.c_int32),
-        ("rowmap", ctypes.c_void_p),
+        ("rowmap", ctypes.c_void_p), ("stream_rows_over", ctypes.c_int32),
     ]
 
 

@@ -851,13 +851,18 @@ int launch_gather(const GatherArgs<T> &a, hipStream_t stream) {
     return launch_gather_lpr<T, 1, OP>(a, stream);
 }
 
-template <typename T>
-__global__ void divide_counts_kernel(T *reps, const int32_t *counts, int64_t groups, int64_t F) {
-    const int64_t n = groups * F;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-         i += (int64_t)gridDim.x * blockDim.x) {
-        int c = counts[i / F];
-        reps[i] = reps[i] / (T)max(c, 1);
+// reps[g, :] /= max(counts[g], 1), VEC features per thread (a row holds `slots` such pieces).
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void divide_counts_kernel(T *reps, const int32_t *counts, int64_t total_slots,
+                                                              uint32_t slots) {
+    const bool narrow = total_slots < ((int64_t)1 << 32);  // the row of a piece by a 32-bit division
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total_slots; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t g = narrow ? (int64_t)((uint32_t)i / slots) : i / (int64_t)slots;
+        const T c = (T)max(counts[g], 1);
+        LPack<T, VEC> v = *reinterpret_cast<const LPack<T, VEC> *>(reps + i * VEC);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) v.v[k] = v.v[k] / c;
+        *reinterpret_cast<LPack<T, VEC> *>(reps + i * VEC) = v;
     }
 }
 
@@ -1006,12 +1011,19 @@ extern "C" size_t cgnn_cluster_mean_workspace_bytes(int64_t N, int64_t F, int64_
 template <typename T>
 static int divide_counts(void *reps, const int32_t *counts, int64_t groups, int64_t F,
                          hipStream_t stream) {
-    const int64_t n = groups * F;
-    if (n == 0) return CGNN_OK;
-    int64_t blocks = ceil_div(n, kBlock);
-    if (blocks > 16384) blocks = 16384;
-    hipLaunchKernelGGL(divide_counts_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
-                       static_cast<T *>(reps), counts, groups, F);
+    if (groups * F == 0) return CGNN_OK;
+    constexpr int WIDE = 16 / sizeof(T);
+    const bool wide = F % WIDE == 0 && reinterpret_cast<uintptr_t>(reps) % 16 == 0;
+    const int64_t slots = wide ? F / WIDE : F, total = groups * slots;
+    if (slots >= ((int64_t)1 << 32)) return fail(CGNN_EUNSUPPORTED, "cluster_mean: rows too wide");
+    int64_t blocks = ceil_div(total, kBlock);
+    if (blocks > 65536) blocks = 65536;
+    if (wide)
+        hipLaunchKernelGGL((divide_counts_kernel<T, WIDE>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                           static_cast<T *>(reps), counts, total, (uint32_t)slots);
+    else
+        hipLaunchKernelGGL((divide_counts_kernel<T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                           static_cast<T *>(reps), counts, total, (uint32_t)slots);
     return check_launch("divide_counts");
 }
 

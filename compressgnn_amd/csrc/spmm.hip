@@ -88,6 +88,7 @@ struct SpmmArgs {
     int32_t stretch_log2;  // log2 of the workgroups per XCD stretch (see logical_block); set at launch
     int32_t blocks;        // workgroups with work (the grid rounds this up to a multiple of kXcds)
     int32_t read_once;     // MODE_UNIT: every row of X is gathered once (member lists), so with streaming loads
+    int32_t stream_over;   // nnz schedule: runs inside a row of more entries than this gather with streaming loads (0: none)
 };
 
 // carry_row values below zero: the run carries nothing, or its carry was added to that
@@ -223,7 +224,7 @@ __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_
 // Gather one feature tile of column c (source chosen by `src` in MODE_DUAL, masked by
 // M in MODE_RELU_MASK).
 template <typename T, int VEC, int MODE>
-__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int src, int64_t foff) {
+__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int src, int64_t foff, bool stream = false) {
     Pack<T, VEC> x;
     if (foff < 0) {
 #pragma unroll
@@ -239,7 +240,8 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
     }
     const int64_t off = (int64_t)c * (int32_t)a.F + foff;  // F < 2^31: one 32 x 32 -> 64 bit multiply
     // rows that are gathered once (member lists; masks exist for those only) are not kept in the caches
-    if (MODE == MODE_RELU_MASK || (MODE == MODE_UNIT && a.read_once)) x = load_pack_stream<T, VEC>(base + off);
+    // (`stream`: the same for the runs of hub rows of a graph block when the block asks for it; uniform over the wave)
+    if (MODE == MODE_RELU_MASK || (MODE == MODE_UNIT && a.read_once) || stream) x = load_pack_stream<T, VEC>(base + off);
     else x = load_pack<T, VEC>(base + off);
     if constexpr (MODE == MODE_RELU_MASK) {
         Pack<T, VEC> m = load_pack_stream<T, VEC>(a.M + off);
@@ -428,6 +430,17 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     acc.clear();
     int cur = -1;
     bool continues = false;
+    // Hub rows: when every run of this wave lies inside a row of more than stream_over entries,
+    // its gathers do not displace lines that the short rows around them come back to.
+    bool stream = false;
+    if (a.stream_over > 0) {
+        bool hub = true;
+        if (active) {
+            const int first = a.rowidx[e0];
+            hub = first == a.rowidx[e1 - 1] && a.rowptr[first + 1] - a.rowptr[first] > a.stream_over;
+        }
+        stream = __ballot(!hub) == 0;
+    }
     if (active) {
         cur = a.rowidx[e0];
         if constexpr (LPR >= kUnroll && sizeof(T) == 4) {
@@ -472,7 +485,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                             if (u0 + u < cnt) {
 #pragma unroll
                                 for (int t = 0; t < TILES; ++t)
-                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
+                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t], stream);
                             }
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u) {
@@ -1000,6 +1013,7 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     if (mode != MODE_DUAL) split = INT32_MAX;  // every column comes from X
     SpmmArgs<T> a = make_args<T>(A, X, X1, split, M, Y, F, accumulate);
     a.read_once = mode == MODE_UNIT || mode == MODE_RELU_MASK;  // asked for by name: the cluster reductions
+    a.stream_over = A->stream_rows_over > 0 ? A->stream_rows_over : 0;
     kernel = resolve_kernel(A, kernel);
     if (mode == MODE_RELU_MASK) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
     if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;

@@ -64,6 +64,7 @@ struct DeviceCsr {
     Tensor rowmap;  // optional: stored row g is output row rowmap[g]
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
+    int32_t stream_rows_over = 0;
     std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
 
     cgnn_csr view() const {
@@ -78,6 +79,7 @@ struct DeviceCsr {
         a.max_row_nnz = max_row_nnz;
         a.seg_nnz = seg_nnz;
         a.rowmap = rowmap.defined() ? rowmap.data_ptr<int32_t>() : nullptr;
+        a.stream_rows_over = stream_rows_over;
         return a;
     }
 
@@ -722,6 +724,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def_readonly("nnz", &DeviceCsr::nnz)
         .def_readonly("max_row_nnz", &DeviceCsr::max_row_nnz)
         .def_readwrite("seg_nnz", &DeviceCsr::seg_nnz)
+        .def_readwrite("stream_rows_over", &DeviceCsr::stream_rows_over)
         .def_readonly("rowptr", &DeviceCsr::rowptr)
         .def_readonly("colidx", &DeviceCsr::colidx)
         .def_readonly("rowidx", &DeviceCsr::rowidx)

@@ -66,6 +66,11 @@ typedef struct cgnn_csr {
      * of such a block are numbered so that consecutive stored rows land on the same XCD
      * (the eight L2 caches of an MI355X are private). */
     const int32_t *rowmap; /* [rows] or NULL */
+    /* NNZ schedule, optional (0 = off): runs that lie inside a row of more than this many
+     * entries gather their rows of X with streaming loads, so that a hub row's gathers are
+     * not kept in the L2 caches.  Pays only where the rows a hub gathers are not gathered again
+     * soon by other rows; results are unchanged. */
+    int32_t stream_rows_over;
 } cgnn_csr;
 
 const char *cgnn_last_error(void);
