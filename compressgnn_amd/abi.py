@@ -27,6 +27,8 @@ EXPORTS = [
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
     "cgnn_cluster_mean_workspace_bytes", "cgnn_cluster_mean", "cgnn_cluster_mean_backward",
     "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_copy_bytes", "cgnn_read_bytes", "cgnn_fill_bytes",
+    "cgnn_exclusive_sum_workspace_bytes", "cgnn_exclusive_sum_i32", "cgnn_sample_count", "cgnn_sample_fill",
+    "cgnn_sample_relabel_begin", "cgnn_sample_relabel_workspace_bytes", "cgnn_sample_relabel",
 ]
 
 
@@ -53,7 +55,8 @@ def lib():
         L.cgnn_version.restype = ctypes.c_char_p
         for name in ("cgnn_spmm_workspace_bytes", "cgnn_spmm_static_scratch_bytes", "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_group_workspace_bytes",
                      "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_mean_workspace_bytes",
-                     "cgnn_csr_transpose_workspace_bytes", "cgnn_compress_batch_workspace_bytes"):
+                     "cgnn_csr_transpose_workspace_bytes", "cgnn_compress_batch_workspace_bytes",
+                     "cgnn_exclusive_sum_workspace_bytes", "cgnn_sample_relabel_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
         _lib = L
     return _lib

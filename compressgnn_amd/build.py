@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 LIB_DIR = os.path.join(HERE, "lib")
 
-HIP_SOURCES = ["spmm.hip", "cluster.hip", "cluster_sort.hip", "transpose.hip", "merger.hip", "abi.cpp"]
+HIP_SOURCES = ["spmm.hip", "cluster.hip", "cluster_sort.hip", "transpose.hip", "merger.hip", "sample.hip", "abi.cpp"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # products and sums are rounded separately so that row sums match a sequential

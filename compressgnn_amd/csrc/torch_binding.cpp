@@ -685,6 +685,150 @@ std::tuple<Tensor, Tensor, c10::optional<Tensor>> csr_transpose(Tensor rowptr, T
     return {colptr, row, c10::nullopt};
 }
 
+// ------------------------------------------------ neighbour sampling (compressed graph) ----
+
+// The host side of a sampling call: sizes the outputs of every layer (two scalar reads per
+// layer: neighbours of the layer, vertices it adds) and strings the device entry points
+// together.  neighbor_sample_sim_impl / neighbor_sample_ori_impl of the reference's module
+// compressgnn_sample (src/sample/csrc/neighbor_sample.h:27-131, 134-211), on GPU tensors.
+struct SampleGraph {
+    cgnn_sample_graph view{};
+    std::vector<Tensor> keep;  // contiguous int64 tensors behind the pointers
+    torch::Device device = torch::kCPU;
+
+    const int64_t *hold(const Tensor &t, const char *name) {
+        TORCH_CHECK(t.defined() && t.is_cuda() && t.scalar_type() == torch::kInt64 && t.dim() == 1,
+                    "neighbor_sample: ", name, " has to be a one-dimensional int64 GPU tensor");
+        TORCH_CHECK(keep.empty() || t.device() == device, "neighbor_sample: ", name, " lives on another device");
+        device = t.device();
+        keep.push_back(t.contiguous());
+        return keep.back().numel() ? keep.back().data_ptr<int64_t>() : nullptr;
+    }
+};
+
+std::tuple<Tensor, Tensor, Tensor> run_sampler(SampleGraph &G, const Tensor &input_node,
+                                               const std::vector<int64_t> &num_neighbors, int64_t seed, bool swap_roles) {
+    const char *op = "neighbor_sample";
+    const cgnn_sample_graph &g = G.view;
+    TORCH_CHECK(input_node.is_cuda() && input_node.device() == G.device && input_node.scalar_type() == torch::kInt64 &&
+                    input_node.dim() == 1,
+                op, ": input_node has to be a one-dimensional int64 tensor beside the graph");
+    for (int64_t fan : num_neighbors) TORCH_CHECK(fan >= 0, op, ": a fan-out of ", fan);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(G.device);
+    auto stream = current_stream(input_node);
+    auto i64 = input_node.options();
+    auto i32 = input_node.options().dtype(torch::kInt32);
+    auto u8 = input_node.options().dtype(torch::kUInt8);
+    const Tensor input = input_node.contiguous();
+    const int64_t n_input = input.numel();
+    Tensor local_of = torch::empty({std::max<int64_t>(g.vertex_cnt, 1)}, i32), seen_at = torch::empty_like(local_of);
+    Tensor status = torch::empty({1}, i32);
+    ok(cgnn_sample_relabel_begin(g.vertex_cnt, n_input, n_input ? input.data_ptr<int64_t>() : nullptr,
+                                 local_of.data_ptr<int32_t>(), seen_at.data_ptr<int32_t>(), status.data_ptr<int32_t>(),
+                                 stream),
+       op);
+    auto raise_on = [&](int32_t code) {
+        TORCH_CHECK_INDEX(code != CGNN_SAMPLE_OUT_OF_RANGE, "Neighbor index out of range");
+        TORCH_CHECK(code != CGNN_SAMPLE_BAD_VERTEX, op, ": a vertex id outside [0, ", g.vertex_cnt, ")");
+        TORCH_CHECK(code != CGNN_SAMPLE_TOO_MANY, op, ": a layer of more than 2^31 - 2 neighbours");
+    };
+    Tensor samples = input.clone();
+    std::vector<Tensor> sources, numbers;
+    int64_t begin = 0, end = n_input;
+    for (size_t layer = 0; layer < num_neighbors.size(); ++layer) {
+        const int64_t n = end - begin, fanout = num_neighbors[layer];
+        if (n == 0) break;
+        Tensor frontier = samples.narrow(0, begin, n);
+        Tensor counts = torch::empty({n}, i32), offsets = torch::empty({n + 1}, i32);
+        ok(cgnn_sample_count(&g, n, frontier.data_ptr<int64_t>(), fanout, counts.data_ptr<int32_t>(),
+                             status.data_ptr<int32_t>(), stream),
+           op);
+        const size_t sum_bytes = cgnn_exclusive_sum_workspace_bytes(n);
+        Tensor sum_ws = torch::empty({(int64_t)std::max<size_t>(sum_bytes, 1)}, u8);
+        ok(cgnn_exclusive_sum_i32(n, counts.data_ptr<int32_t>(), offsets.data_ptr<int32_t>(), status.data_ptr<int32_t>(),
+                                  sum_ws.data_ptr(), sum_bytes, stream),
+           op);
+        // first scalar read of the layer: its size (and whether anything went wrong so far)
+        Tensor head = torch::stack({offsets[n], status[0]}).cpu();
+        raise_on(head.data_ptr<int32_t>()[1]);
+        const int64_t total = head.data_ptr<int32_t>()[0];
+        Tensor neighbors = torch::empty({total}, i64), source = torch::empty({total}, i64), picks = torch::empty({total}, i64);
+        Tensor number = torch::empty({total}, i64), added = torch::empty({1}, i64);
+        Tensor grown = torch::empty({end + total}, i64);
+        grown.narrow(0, 0, end).copy_(samples);
+        if (total > 0) {
+            ok(cgnn_sample_fill(&g, n, frontier.data_ptr<int64_t>(), fanout, offsets.data_ptr<int32_t>(), begin,
+                                (int64_t)layer, (uint64_t)seed, neighbors.data_ptr<int64_t>(), source.data_ptr<int64_t>(),
+                                picks.data_ptr<int64_t>(), status.data_ptr<int32_t>(), stream),
+               op);
+        }
+        const size_t bytes = cgnn_sample_relabel_workspace_bytes(total);
+        Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, u8);
+        ok(cgnn_sample_relabel(total, total ? neighbors.data_ptr<int64_t>() : nullptr, end, local_of.data_ptr<int32_t>(),
+                               seen_at.data_ptr<int32_t>(), grown.data_ptr<int64_t>(), total ? number.data_ptr<int64_t>() : nullptr,
+                               added.data_ptr<int64_t>(), ws.data_ptr(), bytes, stream),
+           op);
+        // second scalar read: how many vertices the layer added
+        Tensor tail = torch::stack({added[0], status[0].to(torch::kInt64)}).cpu();
+        raise_on((int32_t)tail.data_ptr<int64_t>()[1]);
+        const int64_t fresh = tail.data_ptr<int64_t>()[0];
+        samples = grown.narrow(0, 0, end + fresh);
+        sources.push_back(source);
+        numbers.push_back(number);
+        begin = end;
+        end += fresh;
+    }
+    Tensor empty = torch::empty({0}, i64);
+    Tensor of_source = sources.empty() ? empty : torch::cat(sources), of_neighbor = numbers.empty() ? empty : torch::cat(numbers);
+    // (samples, rows, cols): the compressed form reports (source, neighbour), the plain form the reverse
+    if (swap_roles) return {samples.clone(), of_neighbor, of_source};
+    return {samples.clone(), of_source, of_neighbor};
+}
+
+std::tuple<Tensor, Tensor, Tensor> neighbor_sample_cg_sim(Tensor v2v_vlist, Tensor v2v_elist, Tensor v2r_vlist,
+                                                          Tensor v2r_elist, Tensor r2v_vlist, Tensor r2v_elist,
+                                                          std::vector<Tensor> r2r_vlist, std::vector<Tensor> r2r_elist,
+                                                          Tensor v_degree, Tensor r_degree, Tensor input_node,
+                                                          std::vector<int64_t> num_neighbors, int64_t seed) {
+    SampleGraph G;
+    cgnn_sample_graph &g = G.view;
+    g.v2v_ptr = G.hold(v2v_vlist, "v2v_vlist");
+    g.v2v_idx = G.hold(v2v_elist, "v2v_elist");
+    g.v2r_ptr = G.hold(v2r_vlist, "v2r_vlist");
+    g.v2r_idx = G.hold(v2r_elist, "v2r_elist");
+    g.r2v_ptr = G.hold(r2v_vlist, "r2v_vlist");
+    g.r2v_idx = G.hold(r2v_elist, "r2v_elist");
+    TORCH_CHECK(r2r_vlist.size() == r2r_elist.size() && r2r_vlist.size() <= CGNN_SAMPLE_MAX_LEVELS,
+                "neighbor_sample: ", r2r_vlist.size(), " row-pointer and ", r2r_elist.size(), " column tensors of rule levels (at most ",
+                CGNN_SAMPLE_MAX_LEVELS, " levels)");
+    g.levels = (int32_t)r2r_vlist.size();
+    g.vertex_cnt = v2v_vlist.numel() - 1;
+    g.rule_cnt = r2v_vlist.numel() - 1;
+    TORCH_CHECK(g.vertex_cnt >= 0 && g.rule_cnt >= 0 && v2r_vlist.numel() == g.vertex_cnt + 1,
+                "neighbor_sample: row pointers have to hold vertex_cnt + 1 (v2v, v2r) and rule_cnt + 1 (r2v) entries");
+    for (int k = 0; k < g.levels; ++k) {
+        TORCH_CHECK(r2r_vlist[k].numel() == g.rule_cnt + 1, "neighbor_sample: level ", k, " has to hold rule_cnt + 1 row pointers");
+        g.r2r_ptr[k] = G.hold(r2r_vlist[k], "r2r_vlist");
+        g.r2r_idx[k] = G.hold(r2r_elist[k], "r2r_elist");
+    }
+    TORCH_CHECK(v_degree.numel() == g.vertex_cnt && r_degree.numel() == g.rule_cnt,
+                "neighbor_sample: one expanded degree per vertex and per rule");
+    g.v_degree = G.hold(v_degree, "v_degree");
+    g.r_degree = G.hold(r_degree, "r_degree");
+    return run_sampler(G, input_node, num_neighbors, seed, false);
+}
+
+std::tuple<Tensor, Tensor, Tensor> neighbor_sample_ori_impl(Tensor colptr, Tensor row, Tensor input_node,
+                                                            std::vector<int64_t> num_neighbors, int64_t seed) {
+    SampleGraph G;
+    cgnn_sample_graph &g = G.view;
+    g.v2v_ptr = G.hold(colptr, "colptr");
+    g.v2v_idx = G.hold(row, "row");
+    g.vertex_cnt = colptr.numel() - 1;
+    TORCH_CHECK(g.vertex_cnt >= 0, "neighbor_sample: colptr has to hold vertex_cnt + 1 entries");
+    return run_sampler(G, input_node, num_neighbors, seed, true);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -706,6 +850,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("relu"), py::arg("members") = py::none());
     m.def("cluster_reconstruct_backward", &cluster_reconstruct_backward, py::arg("grad"), py::arg("index"),
           py::arg("output"), py::arg("groups"), py::arg("relu"), py::arg("members") = py::none());
+    // the reference's sampler module (src/sample/csrc/function.cpp:7-9), here on GPU tensors; `seed` keys
+    // the counter-based generator of the random positions
+    m.def("neighbor_sample_cg_sim", &neighbor_sample_cg_sim, "Neighbor Sample with CompressGraph Format",
+          py::arg("v2v_vlist"), py::arg("v2v_elist"), py::arg("v2r_vlist"), py::arg("v2r_elist"), py::arg("r2v_vlist"),
+          py::arg("r2v_elist"), py::arg("r2r_vlist"), py::arg("r2r_elist"), py::arg("v_degree"), py::arg("r_degree"),
+          py::arg("input_node"), py::arg("num_neighbors"), py::arg("seed") = 0);
+    m.def("neighbor_sample_ori_impl", &neighbor_sample_ori_impl, "Neighbor Sample with Normal Graph Format",
+          py::arg("colptr"), py::arg("row"), py::arg("input_node"), py::arg("num_neighbors"), py::arg("seed") = 0);
     // additions of this build
     m.def("cluster_members", &cluster_members, "member lists (offsets, perm, sorted_id) of the clusters");
     m.def("csr_transpose", &csr_transpose, "CSR -> CSC of an int64 block on the GPU, SparseTensor.csc() order",

@@ -51,6 +51,7 @@ class CompressGraph():
     def __getstate__(self):
         state = dict(self.__dict__)
         state['_plan'] = None
+        state.pop('_sampler_blocks', None)
         return state
 
     def __setstate__(self, state):
@@ -72,6 +73,7 @@ class CompressGraph():
         self.vertex_degree = self.vertex_degree.to(device)
         self.rule_degree = self.rule_degree.to(device)
         self._plan = None
+        self._sampler_blocks = None
         return self
 
     @property

@@ -254,6 +254,82 @@ int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int64_t max_
                               const int32_t *sorted_id, int relu, void *reps_grad,
                               void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
 
+/* ---------------------------------------- neighbour sampling on a compressed graph -- */
+
+/* The work of the reference's CPU module compressgnn_sample
+ * (src/sample/csrc/function.cpp:7-9: neighbor_sample_cg_sim = neighbor_sample_sim_impl,
+ * src/sample/csrc/neighbor_sample.h:27-131, over get_neighbor / get_neighbor_list of
+ * src/sample/csrc/storage_api.h:6-118; neighbor_sample_ori_impl, :134-211, is the graph without
+ * rules) as device entry points.  One layer: cgnn_sample_count -> cgnn_exclusive_sum_i32 ->
+ * (the caller reads the total and sizes the outputs) -> cgnn_sample_fill -> cgnn_sample_relabel;
+ * cgnn_sample_relabel_begin once per call before the first layer. */
+#define CGNN_SAMPLE_MAX_LEVELS 16
+
+/* The blocks of a CompressGraph as the sampler reads them: int64 arrays on the device, the
+ * tensors of loader/compress_graph.py:21-43 (csr() of v2v_graph, v2r_graph, r2v_graph and of
+ * every r2r level, vertex_degree, rule_degree).  A graph without rules (rule_cnt = 0, levels = 0)
+ * may leave everything but v2v_ptr / v2v_idx NULL: v2v is then (colptr, row) and the degree of
+ * a vertex is the length of its row. */
+typedef struct cgnn_sample_graph {
+    int64_t vertex_cnt, rule_cnt;
+    int32_t levels;                       /* r2r levels, at most CGNN_SAMPLE_MAX_LEVELS */
+    const int64_t *v2v_ptr, *v2v_idx;     /* [vertex_cnt + 1], [nnz] */
+    const int64_t *v2r_ptr, *v2r_idx;     /* [vertex_cnt + 1], [nnz]: rules in [0, rule_cnt) */
+    const int64_t *r2v_ptr, *r2v_idx;     /* [rule_cnt + 1], [nnz] */
+    const int64_t *r2r_ptr[CGNN_SAMPLE_MAX_LEVELS]; /* [rule_cnt + 1] per level */
+    const int64_t *r2r_idx[CGNN_SAMPLE_MAX_LEVELS];
+    const int64_t *v_degree, *r_degree;   /* expanded degrees (gen_degree.h:10-85) */
+} cgnn_sample_graph;
+
+/* *status (device int32; cleared by cgnn_sample_relabel_begin) after the kernels of a call: */
+enum cgnn_sample_status {
+    CGNN_SAMPLE_OK = 0,
+    CGNN_SAMPLE_OUT_OF_RANGE = 1, /* a random position beyond what the descent through the rules finds:
+                                     where the reference throws std::out_of_range (storage_api.h:69) */
+    CGNN_SAMPLE_BAD_VERTEX = 2,   /* a vertex id outside [0, vertex_cnt) in the input or in the graph */
+    CGNN_SAMPLE_TOO_MANY = 3      /* more than 2^31 - 2 neighbours in one layer */
+};
+
+/* out[0] = 0, out[i + 1] = in[0] + ... + in[i]: n + 1 entries.  A sum beyond 2^31 - 2 is
+ * stored as INT32_MAX and reported through *status (may be NULL). */
+size_t cgnn_exclusive_sum_workspace_bytes(int64_t n);
+int cgnn_exclusive_sum_i32(int64_t n, const int32_t *in, int32_t *out, int32_t *status, void *workspace,
+                           size_t workspace_bytes, cgnn_stream_t stream);
+
+/* counts[i] = number of neighbours that frontier vertex i contributes to the layer: 0 for a
+ * vertex of degree 0, the length of its full neighbour list when fanout >= its degree, else
+ * fanout (neighbor_sample.h:88-99). */
+int cgnn_sample_count(const cgnn_sample_graph *graph, int64_t n, const int64_t *frontier, int64_t fanout,
+                      int32_t *counts, int32_t *status, cgnn_stream_t stream);
+
+/* Writes the neighbours of frontier vertex i to neighbors[offsets[i] .. offsets[i + 1]) and
+ * first_position + i (its position among the samples) to the same range of sources.  A full
+ * list comes in the order of get_neighbor_list (storage_api.h:72-118); a sampled one holds the
+ * neighbours at the positions the selection loop of neighbor_sample.h:112-118 picks, in the
+ * order it picks them, each resolved as get_neighbor does (storage_api.h:6-70).  The loop's
+ * draws come from a counter-based generator keyed by (seed, layer, first_position + i, step).
+ * picks: scratch of offsets[n] entries. */
+int cgnn_sample_fill(const cgnn_sample_graph *graph, int64_t n, const int64_t *frontier, int64_t fanout,
+                     const int32_t *offsets, int64_t first_position, int64_t layer, uint64_t seed,
+                     int64_t *neighbors, int64_t *sources, int64_t *picks, int32_t *status,
+                     cgnn_stream_t stream);
+
+/* Start of a sampling call: clears *status, marks every vertex as not yet numbered
+ * (local_of and seen_at: int32[vertex_cnt] each) and numbers the input vertices 0, 1, ... (of
+ * equal ones the first counts, as the hash map of neighbor_sample.h:72-76 has it). */
+int cgnn_sample_relabel_begin(int64_t vertex_cnt, int64_t n_input, const int64_t *input, int32_t *local_of,
+                              int32_t *seen_at, int32_t *status, cgnn_stream_t stream);
+
+/* Local numbers for the `total` neighbours of a layer (neighbor_sample.h:100-106,119-125): a
+ * vertex numbered before keeps its number; the others take base, base + 1, ... in the order
+ * of their first occurrence and are appended to samples at those positions (samples needs room
+ * for base + total entries).  numbers[t] = local number of neighbors[t]; *new_count (device) =
+ * vertices added. */
+size_t cgnn_sample_relabel_workspace_bytes(int64_t total);
+int cgnn_sample_relabel(int64_t total, const int64_t *neighbors, int64_t base, int32_t *local_of,
+                        int32_t *seen_at, int64_t *samples, int64_t *numbers, int64_t *new_count,
+                        void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
+
 /* --------------------------------------------------------------- utilities ---- */
 
 /* A plain device-to-device copy kernel of n bytes (n % 16 == 0); the calibration

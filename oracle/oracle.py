@@ -184,3 +184,90 @@ def reconstruct_backward(grad, index, output, groups, relu=False):
     fn(ctypes.c_int64(N), ctypes.c_int64(F), ctypes.c_int64(groups), _ptr(grad), _ptr(output), _ptr(index),
        ctypes.c_int(bool(relu)), _ptr(reps_grad))
     return reps_grad
+
+
+# ---- neighbour sampling over a compressed graph (oracle_sample.c) -------------------------
+DRAW_FN = ctypes.CFUNCTYPE(ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                           ctypes.c_void_p)
+
+
+def _graph_args(blocks):
+    """blocks: dict with v2v, v2r, r2v = (ptr, idx) int64 arrays, r2r = [(ptr, idx), ...],
+    v_degree, r_degree (int64 arrays or None).  Returns (ctypes arguments, keep-alive list)."""
+    keep = []
+
+    def arr(a):
+        a = _c(a, np.int64)
+        keep.append(a)
+        return _ptr(a)
+
+    levels = len(blocks["r2r"])
+    ptrs = (ctypes.c_void_p * max(levels, 1))(*[arr(p).value for p, _ in blocks["r2r"]])
+    idxs = (ctypes.c_void_p * max(levels, 1))(*[arr(i).value if len(i) else None for _, i in blocks["r2r"]])
+    keep += [ptrs, idxs]
+    args = [arr(blocks["v2v"][0]), arr(blocks["v2v"][1]), arr(blocks["v2r"][0]), arr(blocks["v2r"][1]),
+            arr(blocks["r2v"][0]), arr(blocks["r2v"][1]), ctypes.c_int(levels), ptrs, idxs]
+    return args, keep
+
+
+def _take64(pointer, n):
+    out = np.ctypeslib.as_array(pointer, shape=(max(n, 1),))[:n].copy() if n else np.zeros(0, np.int64)
+    lib().oracle_free(pointer)
+    return out
+
+
+def neighbor_sample(blocks, input_node, num_neighbors, draw=None, seed=0, plain=False):
+    """neighbor_sample_cg_sim (src/sample/csrc/neighbor_sample.h:27-131) or, with plain=True and
+    blocks["v2v"] = (colptr, row), neighbor_sample_ori_impl (:134-211).  draw(high) -> int in
+    [0, high): the source of the random indices, called in the reference's order (its
+    uniform_randint, :10-15); None: the counter-based generator of the HIP sampler with `seed`.
+    Returns (samples, rows, cols); raises IndexError where the reference throws out_of_range."""
+    L = lib()
+    if plain:
+        blocks = dict(v2v=blocks["v2v"], v2r=(np.zeros(len(blocks["v2v"][0]), np.int64), np.zeros(0, np.int64)),
+                      r2v=(np.zeros(1, np.int64), np.zeros(0, np.int64)), r2r=[], v_degree=None, r_degree=None)
+    args, keep = _graph_args(blocks)
+    vdeg = _c(blocks["v_degree"] if blocks.get("v_degree") is not None else np.zeros(1), np.int64)
+    rdeg = _c(blocks["r_degree"] if blocks.get("r_degree") is not None else np.zeros(1), np.int64)
+    inp = _c(input_node, np.int64)
+    fan = _c(num_neighbors, np.int64)
+    cb = DRAW_FN(lambda high, layer, i, j, user: int(draw(high))) if draw is not None else ctypes.cast(None, DRAW_FN)
+    ps, pr, pc = (ctypes.POINTER(ctypes.c_int64)() for _ in range(3))
+    ns, ne = ctypes.c_int64(0), ctypes.c_int64(0)
+    vertex_cnt = len(blocks["v2v"][0]) - 1
+    rc = L.oracle_neighbor_sample(ctypes.c_int64(vertex_cnt), *args, _ptr(vdeg), _ptr(rdeg), _ptr(inp),
+                                  ctypes.c_int64(len(inp)), _ptr(fan), ctypes.c_int(len(fan)), ctypes.c_int(1 if plain else 0),
+                                  cb, None, ctypes.c_uint64(seed), ctypes.byref(ps), ctypes.byref(ns), ctypes.byref(pr),
+                                  ctypes.byref(pc), ctypes.byref(ne))
+    samples, rows, cols = _take64(ps, ns.value), _take64(pr, ne.value), _take64(pc, ne.value)
+    if rc != 0:
+        raise IndexError("Neighbor index out of range")
+    return samples, rows, cols
+
+
+def get_neighbors(blocks, nodes, indices):
+    """get_neighbor (src/sample/csrc/storage_api.h:6-70) for (node, index) pairs; -1 where the
+    reference throws out_of_range."""
+    args, keep = _graph_args(blocks)
+    nodes, indices = _c(nodes, np.int64), _c(indices, np.int64)
+    out = np.zeros(len(nodes), np.int64)
+    lib().oracle_get_neighbors(*args, _ptr(_c(blocks["v_degree"], np.int64)), _ptr(_c(blocks["r_degree"], np.int64)),
+                               ctypes.c_int64(len(nodes)), _ptr(nodes), _ptr(indices), _ptr(out))
+    return out
+
+
+def neighbor_list(blocks, node):
+    """get_neighbor_list (src/sample/csrc/storage_api.h:72-118)."""
+    args, keep = _graph_args(blocks)
+    p = ctypes.POINTER(ctypes.c_int64)()
+    L = lib()
+    L.oracle_neighbor_list.restype = ctypes.c_int64
+    n = L.oracle_neighbor_list(*args, ctypes.c_int64(node), ctypes.byref(p))
+    return _take64(p, n)
+
+
+def counter_draw(seed, layer, i, j, high):
+    L = lib()
+    L.oracle_counter_draw.restype = ctypes.c_int64
+    return L.oracle_counter_draw(ctypes.c_uint64(seed), ctypes.c_int64(layer), ctypes.c_int64(i), ctypes.c_int64(j),
+                                 ctypes.c_int64(high))

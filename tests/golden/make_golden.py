@@ -13,6 +13,12 @@ code (oracle/_ref, built by `make -C oracle ref` where the reference checkout ex
                        gen_degree, filter_csr, depth_filter_csr, gen_vertex_order_csr/csc
                        on seeded compressed graphs (inputs are stored with the outputs)
 
+  sample_golden.npz    (samples, rows, cols) of the reference's neighbor_sample_cg_sim and
+                       neighbor_sample_ori_impl on the compressed graphs of offline_golden.npz
+                       (their blocks and expanded degrees are read from that file), with the
+                       seed of torch's CPU generator the reference drew its random positions
+                       from; also which calls raised IndexError (std::out_of_range)
+
 Fixtures hold data only (inputs and expected outputs).  Run from the repository root:
     python tests/golden/make_golden.py
 """
@@ -206,9 +212,52 @@ def make_offline():
     np.savez_compressed(os.path.join(HERE, "offline_golden.npz"), **out)
 
 
+def make_sample():
+    import compressgnn_sample_ref as sampler
+    g = np.load(os.path.join(HERE, "offline_golden.npz"))
+    t = torch.from_numpy
+    out, case = {}, 0
+    rng = np.random.default_rng(77)
+    for i in range(int(g["n_rule_graphs"])):
+        pre = "r%d_" % i
+        V, levels = int(g[pre + "V"]), int(g[pre + "levels"])
+        blocks = [t(g[pre + nm + "_" + part].astype(np.int64)) for nm in ("v2v", "v2r", "r2v") for part in ("vlist", "elist")]
+        lv_ptr = [t(g[pre + "lv%d_vlist" % k].astype(np.int64)) for k in range(levels)]
+        lv_idx = [t(g[pre + "lv%d_elist" % k].astype(np.int64)) for k in range(levels)]
+        vdeg, rdeg = t(g[pre + "vertex_degree"].astype(np.int64)), t(g[pre + "rule_degree"].astype(np.int64))
+        for fan in ([2, 2], [10 ** 6], [3, 10 ** 6, 1], [1], []):
+            inp = rng.integers(0, V, size=int(rng.integers(1, 9))).astype(np.int64)
+            seed = int(rng.integers(0, 10 ** 6))
+            key = "s%d_" % case
+            out.update({key + "graph": np.array(i), key + "input": inp, key + "fan": np.array(fan, np.int64),
+                        key + "seed": np.array(seed), key + "plain": np.array(0)})
+            torch.manual_seed(seed)
+            try:
+                res = sampler.neighbor_sample_cg_sim(*blocks, lv_ptr, lv_idx, vdeg, rdeg, t(inp), fan)
+                out.update({key + "raised": np.array(0), key + "samples": res[0].numpy(), key + "rows": res[1].numpy(),
+                            key + "cols": res[2].numpy()})
+            except IndexError:
+                out[key + "raised"] = np.array(1)
+            case += 1
+        # the plain form on the v2v block alone (a CSC of some graph over the same vertices)
+        for fan in ([2, 3], [10 ** 6, 1]):
+            inp = rng.integers(0, V, size=5).astype(np.int64)
+            seed = int(rng.integers(0, 10 ** 6))
+            key = "s%d_" % case
+            torch.manual_seed(seed)
+            res = sampler.neighbor_sample_ori_impl(blocks[0], blocks[1], t(inp), fan)
+            out.update({key + "graph": np.array(i), key + "input": inp, key + "fan": np.array(fan, np.int64),
+                        key + "seed": np.array(seed), key + "plain": np.array(1), key + "raised": np.array(0),
+                        key + "samples": res[0].numpy(), key + "rows": res[1].numpy(), key + "cols": res[2].numpy()})
+            case += 1
+    out["n_cases"] = np.array(case)
+    np.savez_compressed(os.path.join(HERE, "sample_golden.npz"), **out)
+
+
 if __name__ == "__main__":
     make_spmm()
     make_cluster()
     make_offline()
-    for f in ("spmm_golden.npz", "cluster_golden.npz", "offline_golden.npz"):
+    make_sample()
+    for f in ("spmm_golden.npz", "cluster_golden.npz", "offline_golden.npz", "sample_golden.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

@@ -66,3 +66,15 @@ def test_runtime_module_has_the_reference_operator_names():
                      torch.zeros(1, 3), "rowbalance", None)
     with pytest.raises(RuntimeError):
         rt.cluster_assign(torch.zeros(3, 4), torch.zeros(4, 2), 2, [])
+
+
+def test_sampler_module_has_the_reference_names():
+    """compressgnn_sample, the module name the reference builds from src/sample
+    (function.cpp:7-9): both functions, GPU tensors only."""
+    import torch
+    import compressgnn_sample as sampler
+    for name in ["neighbor_sample_cg_sim", "neighbor_sample_ori_impl"]:
+        assert callable(getattr(sampler, name)), name
+    ptr = torch.zeros(3, dtype=torch.long)
+    with pytest.raises(RuntimeError, match="GPU"):
+        sampler.neighbor_sample_ori_impl(ptr, torch.zeros(0, dtype=torch.long), torch.zeros(1, dtype=torch.long), [2])

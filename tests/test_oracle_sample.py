@@ -1,0 +1,175 @@
+"""Pins the sampler functions of the CPU oracle (oracle/oracle_sample.c; no GPU needed):
+  * golden (samples, rows, cols) recorded from the reference's compiled module on compressed
+    graphs of up to three rule levels (tests/golden/sample_golden.npz): the oracle, fed from
+    the generator the reference drew from (torch's CPU generator under the recorded seed),
+    reproduces them exactly, for the compressed and the plain form;
+  * the compiled reference itself, where oracle/_ref is built, on larger graphs;
+  * the expansion invariant: get_neighbor over all positions of a vertex and the full list
+    are both the expanded in-list of the vertex (as a multiset), on graphs whose hierarchy the
+    reference's degrees cover (one rule level);
+  * the selection loop: distinct positions, all of them when the fan-out covers the degree,
+    the counter-based generator's draws in range and reproducible."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path[:0] = [os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compressgnn_amd", "layer"),
+                os.path.join(ROOT, "compressgnn_amd", "loader")]
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def golden_blocks(g, i):
+    pre = "r%d_" % i
+    levels = int(g[pre + "levels"])
+    pair = lambda nm: (g[pre + nm + "_vlist"].astype(np.int64), g[pre + nm + "_elist"].astype(np.int64))
+    return dict(v2v=pair("v2v"), v2r=pair("v2r"), r2v=pair("r2v"),
+                r2r=[(g[pre + "lv%d_vlist" % k].astype(np.int64), g[pre + "lv%d_elist" % k].astype(np.int64))
+                     for k in range(levels)],
+                v_degree=g[pre + "vertex_degree"].astype(np.int64), r_degree=g[pre + "rule_degree"].astype(np.int64))
+
+
+def torch_draws(seed):
+    """The reference's uniform_randint (src/sample/csrc/neighbor_sample.h:10-15) on the same generator."""
+    torch.manual_seed(seed)
+    return lambda high: int(torch.randint(0, high, (1,)))
+
+
+def blocks_of(graph):
+    pair = lambda b: tuple(t.cpu().numpy() for t in b.csr()[:2])
+    return dict(v2v=pair(graph.v2v_graph), v2r=pair(graph.v2r_graph), r2v=pair(graph.r2v_graph),
+                r2r=[pair(b) for b in graph.r2r_graph], v_degree=graph.vertex_degree.cpu().numpy(),
+                r_degree=graph.rule_degree.cpu().numpy())
+
+
+def compressed(kind, seed=3):
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    if kind == "blocks":
+        n = 64
+        v = np.arange(n + 1, dtype=np.int64) * 32
+        e = np.tile(np.arange(32, dtype=np.int64), n)
+    elif kind == "copy":
+        v, e = off.gen_copy_model(1500, 9.0, 0.7, seed)
+    else:
+        v, e = off.gen_chung_lu(2708, 10500, 2.5, seed)
+    V = len(v) - 1
+    m = np.ones(V, bool)
+    data = CompressgnnData(np.zeros((V, 1), np.float32), (v, e), np.zeros(V, np.int64), m, m, m, graph_type="csr",
+                           min_pair_frequency=3)
+    return data, np.asarray(v, np.int64), np.asarray(e, np.int64)
+
+
+def test_golden_vectors_of_the_compiled_reference():
+    g = np.load(os.path.join(GOLD, "sample_golden.npz"))
+    off = np.load(os.path.join(GOLD, "offline_golden.npz"))
+    assert int(g["n_cases"]) >= 20
+    seen_levels = set()
+    for c in range(int(g["n_cases"])):
+        key = "s%d_" % c
+        blocks = golden_blocks(off, int(g[key + "graph"]))
+        seen_levels.add(len(blocks["r2r"]))
+        plain = bool(g[key + "plain"])
+        run = lambda: oracle.neighbor_sample(blocks, g[key + "input"], g[key + "fan"].tolist(),
+                                             draw=torch_draws(int(g[key + "seed"])), plain=plain)
+        if int(g[key + "raised"]):
+            with pytest.raises(IndexError):
+                run()
+            continue
+        samples, rows, cols = run()
+        assert np.array_equal(samples, g[key + "samples"])
+        assert np.array_equal(rows, g[key + "rows"]) and np.array_equal(cols, g[key + "cols"])
+    assert {0, 1, 3} <= seen_levels
+
+
+@pytest.mark.parametrize("kind", ["blocks", "copy", "chung_lu"])
+def test_matches_the_compiled_reference(kind):
+    ref = pytest.importorskip("compressgnn_sample_ref")
+    data, v, e = compressed(kind)
+    b = blocks_of(data.edge_index)
+    t = torch.from_numpy
+    rng = np.random.default_rng(5)
+    V = data.vertex_cnt
+    for fan in ([3, 2], [10 ** 6, 10 ** 6], [5, 10 ** 6, 2], [1, 1, 1, 1]):
+        inp = rng.integers(0, V, size=12).astype(np.int64)
+        inp[3] = inp[0]  # a vertex given twice
+        seed = int(rng.integers(0, 10 ** 6))
+        torch.manual_seed(seed)
+        want = ref.neighbor_sample_cg_sim(t(b["v2v"][0]), t(b["v2v"][1]), t(b["v2r"][0]), t(b["v2r"][1]), t(b["r2v"][0]),
+                                          t(b["r2v"][1]), [t(p) for p, _ in b["r2r"]], [t(i) for _, i in b["r2r"]],
+                                          t(b["v_degree"]), t(b["r_degree"]), t(inp), fan)
+        got = oracle.neighbor_sample(b, inp, fan, draw=torch_draws(seed))
+        for a, w in zip(got, want):
+            assert np.array_equal(a, w.numpy())
+        # the plain form on the uncompressed in-lists of the same graph
+        import compressgnn_offline as off
+        colptr, row, _ = off.csr_transpose(v, e, None, V)
+        torch.manual_seed(seed)
+        want = ref.neighbor_sample_ori_impl(t(colptr), t(row), t(inp), fan)
+        got = oracle.neighbor_sample(dict(v2v=(colptr, row)), inp, fan, draw=torch_draws(seed), plain=True)
+        for a, w in zip(got, want):
+            assert np.array_equal(a, w.numpy())
+
+
+@pytest.mark.parametrize("kind", ["blocks", "copy"])
+def test_expansion_invariant(kind):
+    """Whatever the order, the positions 0 .. degree-1 of a vertex and its full list name the
+    in-neighbours of the vertex in the graph with self loops that was compressed."""
+    import compressgnn_offline as off
+    data, v, e = compressed(kind)
+    assert data.rule_cnt > 0 and data.edge_index.step <= 1
+    b = blocks_of(data.edge_index)
+    v2, e2 = off.add_self_loop_csr(v, e)
+    V = data.vertex_cnt
+    colptr, row, _ = off.csr_transpose(v2, e2, None, V)
+    rng = np.random.default_rng(1)
+    with_rules = np.nonzero(np.diff(b["v2r"][0]))[0]
+    assert len(with_rules)
+    for node in list(rng.integers(0, V, size=25)) + list(with_rules[:15]):
+        want = np.sort(row[colptr[node]:colptr[node + 1]])
+        degree = int(b["v_degree"][node])
+        assert degree == len(want)
+        by_position = oracle.get_neighbors(b, np.full(degree, node), np.arange(degree))
+        assert np.array_equal(np.sort(by_position), want)
+        assert np.array_equal(np.sort(oracle.neighbor_list(b, node)), want)
+        assert oracle.get_neighbors(b, [node], [degree])[0] == -1  # one past the end: the reference throws
+
+
+def test_selection_loop_properties():
+    data, v, e = compressed("copy")
+    b = blocks_of(data.edge_index)
+    V = data.vertex_cnt
+    inp = np.arange(0, V, 7, dtype=np.int64)
+    for fan in (1, 3, 8):
+        samples, rows, cols = oracle.neighbor_sample(b, inp, [fan], seed=9)
+        again = oracle.neighbor_sample(b, inp, [fan], seed=9)
+        assert all(np.array_equal(x, y) for x, y in zip((samples, rows, cols), again))
+        other = oracle.neighbor_sample(b, inp, [fan], seed=10)
+        assert not np.array_equal(other[2], cols)
+        assert np.array_equal(samples[:len(inp)], inp) and len(np.unique(samples)) == len(samples)
+        per_vertex = np.bincount(rows, minlength=len(inp))
+        assert np.array_equal(per_vertex, np.minimum(b["v_degree"][inp], fan))
+        # every sampled neighbour is an in-neighbour, and no position is taken twice: the
+        # neighbours of a vertex without duplicate in-edges are distinct
+        for i in range(0, len(inp), 17):
+            mine = samples[cols[rows == i]]
+            full = oracle.neighbor_list(b, inp[i])
+            assert set(mine) <= set(full)
+            if len(set(full)) == len(full):
+                assert len(set(mine)) == len(mine)
+    # a fan-out that covers every degree returns the full lists in order
+    samples, rows, cols = oracle.neighbor_sample(b, inp[:20], [10 ** 9], seed=1)
+    at = 0
+    for i in range(20):
+        full = oracle.neighbor_list(b, inp[i])
+        assert np.array_equal(samples[cols[at:at + len(full)]], full) and np.all(rows[at:at + len(full)] == i)
+        at += len(full)
+    assert at == len(rows)
+    draws = [oracle.counter_draw(5, 1, 10, j, j) for j in range(1, 200)]
+    assert all(0 <= d < j for d, j in zip(draws, range(1, 200)))
+    assert len(set(oracle.counter_draw(5, 1, i, 1000, 1000) for i in range(100))) > 60
