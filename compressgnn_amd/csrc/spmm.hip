@@ -89,6 +89,9 @@ struct SpmmArgs {
     int32_t blocks;        // workgroups with work (the grid rounds this up to a multiple of kXcds)
     int32_t read_once;     // MODE_UNIT: every row of X is gathered once (member lists), so with streaming loads
     int32_t stream_over;   // nnz schedule: runs inside a row of more entries than this gather with streaming loads (0: none)
+    const int32_t *cut_rows;    // spmm_fixup_rows_kernel: the stored rows that the runs cut, ascending
+    const int32_t *empty_rows;  // and the stored rows without entries
+    int32_t n_cut_rows, n_empty_rows;
 };
 
 // carry_row values below zero: the run carries nothing, or its carry was added to that
@@ -802,6 +805,64 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<T> a) {
     }
 }
 
+// The same pass for a block that comes with the lists of its cut rows and its empty rows
+// (both follow from rowptr and the run length alone, so they are made once per block): a lane
+// group per cut row, and nothing for the many runs that carry nothing.  The carries of a row
+// sit where the nnz kernel's workgroups left them: at the run the row starts in, and at the first
+// run of every following workgroup whose end still lies inside the row; they are added in that
+// (ascending) order, the same as in spmm_fixup_kernel, so the result is the same bit for bit.
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kBlock) void spmm_fixup_rows_kernel(SpmmArgs<T> a) {
+    constexpr int GPB = kBlock / LPR;
+    constexpr int BATCH = 8;
+    const int sub = threadIdx.x % LPR;
+    int item = blockIdx.x * GPB + threadIdx.x / LPR;
+    if constexpr (LPR == kWave) item = __builtin_amdgcn_readfirstlane(item);
+    if (item < a.n_cut_rows) {
+        const int row = a.cut_rows[item];
+        const int64_t row_end = a.rowptr[row + 1];
+        const int64_t s0 = a.rowptr[row] / a.seg_nnz;           // the run the row starts in
+        const int64_t group0 = s0 / a.merge_stride * a.merge_stride;  // first run of that run's workgroup
+#pragma unroll 1
+        for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC) {
+            Pack<T, VEC> acc, zero;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc.v[i] = zero.v[i] = T(0);
+            bool more = true;
+#pragma unroll 1
+            for (int k = 0; more; k += BATCH) {
+                bool take[BATCH];
+                Pack<T, VEC> c[BATCH];
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u) {
+                    const int64_t p = (k + u == 0) ? s0 : group0 + (int64_t)(k + u) * a.merge_stride;
+                    take[u] = (k + u == 0) || (p + 1) * a.seg_nnz < row_end;
+                    c[u] = take[u] ? load_pack<T, VEC>(a.carry + p * a.F + f) : zero;
+                }
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u) {
+                    more = more && take[u];
+                    if (more)
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) acc.v[i] = acc.v[i] + c[u].v[i];
+                }
+            }
+            T *y = a.Y + (int64_t)out_row(a, row) * a.F + f;
+            Pack<T, VEC> o = load_pack<T, VEC>(y);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) o.v[i] = o.v[i] + acc.v[i];
+            store_pack<T, VEC>(y, o);
+        }
+    }
+    if (a.accumulate || item >= a.n_empty_rows) return;
+    const int erow = out_row(a, a.empty_rows[item]);
+    Pack<T, VEC> zero;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) zero.v[i] = T(0);
+    for (int64_t f = (int64_t)sub * VEC; f < a.F; f += (int64_t)LPR * VEC)
+        store_pack_stream<T, VEC>(a.Y + (int64_t)erow * a.F + f, zero);
+}
+
 // ------------------------------------------------------------------- dispatch --
 struct Shape {
     int vec, lpr, tiles, grid_y;
@@ -840,7 +901,7 @@ Shape pick_shape(int64_t F, const void *p0, const void *p1, const void *p2, cons
     return s;
 }
 
-enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2, KIND_REDUCE = 3 };
+enum { KIND_ROW = 0, KIND_NNZ = 1, KIND_FIXUP = 2, KIND_REDUCE = 3, KIND_FIXUP_ROWS = 4 };
 
 template <typename T, int VEC, int LPR, int TILES>
 int launch_shape(int kind, int mode, const SpmmArgs<T> &args, int64_t items, int grid_y, hipStream_t stream) {
@@ -881,6 +942,10 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &args, int64_t items, int
                 hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, LPR, false>), fix_grid, block, 0, stream, a);
             break;
         }
+        case KIND_FIXUP_ROWS:  // items = lane groups: one per cut row, one per empty row
+            hipLaunchKernelGGL((spmm_fixup_rows_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, GPB)), block, 0, stream,
+                               a);
+            break;
         case KIND_REDUCE:  // items = chunks of kCarryFan carries, one lane group each
             hipLaunchKernelGGL((spmm_carry_reduce_kernel<T, VEC, LPR>), dim3((unsigned)ceil_div(items, GPB)), block, 0,
                                stream, a);
@@ -918,15 +983,20 @@ int launch(int kind, int mode, const Shape &s, const SpmmArgs<T> &a, int64_t ite
     return fail(CGNN_EUNSUPPORTED, "spmm: no kernel for this lane layout");
 }
 
+// AUTO: rows are "near regular" when the longest one is a small multiple of the mean;
+// otherwise balance by non-zeros.
+int schedule_for(int64_t rows, int64_t nnz, int32_t max_row_nnz, int kernel) {
+    if (kernel == CGNN_SPMM_ROW || kernel == CGNN_SPMM_NNZ) return kernel;
+    if (max_row_nnz <= 0) return CGNN_SPMM_NNZ;
+    const double mean = rows > 0 ? (double)nnz / (double)rows : 0.0;
+    const double limit = 8.0 * (mean < 8.0 ? 8.0 : mean);
+    return (double)max_row_nnz <= limit ? CGNN_SPMM_ROW : CGNN_SPMM_NNZ;
+}
+
 int resolve_kernel(const cgnn_csr *A, int kernel) {
     if (kernel == CGNN_SPMM_ROW || kernel == CGNN_SPMM_NNZ) return kernel;
-    // AUTO: rows are "near regular" when the longest one is a small multiple of the
-    // mean; otherwise balance by non-zeros.  Needs rowidx for the nnz schedule.
-    if (A->rowidx == nullptr) return CGNN_SPMM_ROW;
-    if (A->max_row_nnz <= 0) return CGNN_SPMM_NNZ;
-    const double mean = A->rows > 0 ? (double)A->nnz / (double)A->rows : 0.0;
-    const double limit = 8.0 * (mean < 8.0 ? 8.0 : mean);
-    return (double)A->max_row_nnz <= limit ? CGNN_SPMM_ROW : CGNN_SPMM_NNZ;
+    if (A->rowidx == nullptr) return CGNN_SPMM_ROW;  // the nnz schedule needs the row of every non-zero
+    return schedule_for(A->rows, A->nnz, A->max_row_nnz, kernel);
 }
 
 int seg_len(const cgnn_csr *A) {
@@ -1064,6 +1134,15 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
         a.carry = level_carries(last);
         a.merge_stride = last == 0 ? runs_per_workgroup : 1;
     }
+    if (A->cut_rows != nullptr && levels.count == 1) {
+        // the block knows which rows its runs cut (and which rows are empty): only those are looked at
+        a.cut_rows = A->cut_rows;
+        a.n_cut_rows = A->n_cut_rows;
+        a.empty_rows = A->empty_rows;
+        a.n_empty_rows = accumulate ? 0 : A->n_empty_rows;
+        const int64_t items = a.n_cut_rows > a.n_empty_rows ? a.n_cut_rows : a.n_empty_rows;
+        return launch<T>(KIND_FIXUP_ROWS, mode, s, a, items, stream);
+    }
     const int64_t items = accumulate ? a.nseg : (a.nseg > A->rows ? a.nseg : A->rows);
     return launch<T>(KIND_FIXUP, mode, s, a, items, stream);
 }
@@ -1154,6 +1233,13 @@ int static_scratch(void **out) {
 }  // namespace cgnn
 
 using namespace cgnn;
+
+extern "C" int cgnn_spmm_schedule(int64_t rows, int64_t nnz, int32_t max_row_nnz, int kernel) {
+    if (kernel < CGNN_SPMM_AUTO || kernel > CGNN_SPMM_NNZ) return CGNN_SPMM_AUTO;
+    return schedule_for(rows, nnz, max_row_nnz, kernel);
+}
+
+extern "C" int cgnn_spmm_run_length(const cgnn_csr *A) { return A == nullptr ? 0 : seg_len(A); }
 
 extern "C" size_t cgnn_spmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
 

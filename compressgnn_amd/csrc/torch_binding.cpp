@@ -65,6 +65,7 @@ struct DeviceCsr {
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
     int32_t stream_rows_over = 0;
+    Tensor cut_rows, empty_rows;  // the rows the runs of the nnz schedule cut / the rows without entries
     std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
 
     cgnn_csr view() const {
@@ -80,10 +81,48 @@ struct DeviceCsr {
         a.seg_nnz = seg_nnz;
         a.rowmap = rowmap.defined() ? rowmap.data_ptr<int32_t>() : nullptr;
         a.stream_rows_over = stream_rows_over;
+        if (cut_rows.defined()) {
+            a.cut_rows = cut_rows.data_ptr<int32_t>();  // a tensor without entries gives a pointer that is never read
+            a.n_cut_rows = (int32_t)cut_rows.numel();
+            a.empty_rows = empty_rows.data_ptr<int32_t>();
+            a.n_empty_rows = (int32_t)empty_rows.numel();
+        }
         return a;
     }
 
+    // Which rows the runs cut depends on rowptr and the run length only: found once, here (two
+    // small host reads at build time), so that the fix-up pass of every product goes straight to them.
+    void list_rows() {
+        cut_rows = Tensor();
+        empty_rows = Tensor();
+        if (rows == 0 || nnz == 0) return;
+        cgnn_csr a = view();
+        const int64_t K = cgnn_spmm_run_length(&a);
+        Tensor start = rowptr.slice(0, 0, rows).to(torch::kInt64), end = rowptr.slice(0, 1, rows + 1).to(torch::kInt64);
+        // a row of at most K entries is never cut; a longer one is cut at the multiples of K inside it
+        Tensor cut = ((end - start) > K).logical_and((torch::floor_divide(start, K) + 1) * K < end);
+        Tensor found = torch::nonzero(cut).flatten().to(torch::kInt32);
+        Tensor none = torch::nonzero(start == end).flatten().to(torch::kInt32);
+        // a pointer is needed even for an empty list (NULL means "no lists"): keep one entry of storage
+        auto pad = [](const Tensor &t) { return t.numel() ? t : torch::zeros({1}, t.options()).narrow(0, 0, 0); };
+        cut_rows = pad(found.contiguous());
+        empty_rows = pad(none.contiguous());
+    }
+
+    // rowidx (the row of every non-zero, as large as colidx) is read by the nnz schedule only:
+    // it is made when a product first resolves to that schedule, on the product's stream.
+    void ensure_rowidx(int kernel) {
+        if (nnz == 0 || rowidx.defined()) return;
+        if (cgnn_spmm_schedule(rows, nnz, max_row_nnz, kernel) != CGNN_SPMM_NNZ) return;
+        rowidx = torch::empty({nnz}, rowptr.options());
+        ok(cgnn_csr_expand_rows(rows, nnz, rowptr.data_ptr<int32_t>(), rowidx.data_ptr<int32_t>(),
+                                reinterpret_cast<cgnn_stream_t>(
+                                    c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(rowptr.device().index()).stream())),
+           "csr_expand_rows");
+    }
+
     Tensor workspace(int64_t F, int dtype, int kernel, size_t *bytes) {
+        ensure_rowidx(kernel);
         cgnn_csr a = view();
         *bytes = cgnn_spmm_workspace_bytes(&a, F, dtype, kernel);
         return scratch->get(*bytes, rowptr);
@@ -93,7 +132,7 @@ struct DeviceCsr {
 // rowptr/col: int64 or int32 tensors on any device; value: float tensor or undefined.
 std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows,
                                     int64_t cols, torch::Device device, int64_t seg_nnz,
-                                    c10::optional<Tensor> rowmap = c10::nullopt) {
+                                    c10::optional<Tensor> rowmap = c10::nullopt, bool with_row_lists = true) {
     TORCH_CHECK(device.is_cuda(), "DeviceCsr lives on a GPU");
     TORCH_CHECK(rowptr.dim() == 1 && col.dim() == 1 && rowptr.numel() == rows + 1, "rowptr must have rows+1 entries");
     auto blk = std::make_shared<DeviceCsr>();
@@ -110,21 +149,16 @@ std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Ten
     if (rp.scalar_type() == torch::kInt64) {
         blk->rowptr = torch::empty({rows + 1}, i32);
         blk->colidx = torch::empty({blk->nnz}, i32);
-        blk->rowidx = torch::empty({blk->nnz}, i32);
         TORCH_CHECK(ci.scalar_type() == torch::kInt64, "rowptr and col must have the same integer type");
         ok(cgnn_csr_prepare_i64(rows, blk->nnz, rp.data_ptr<int64_t>(), blk->nnz ? ci.data_ptr<int64_t>() : nullptr,
                                 blk->rowptr.data_ptr<int32_t>(), blk->nnz ? blk->colidx.data_ptr<int32_t>() : nullptr,
-                                blk->nnz ? blk->rowidx.data_ptr<int32_t>() : nullptr, current_stream(rp)),
+                                nullptr, current_stream(rp)),
            "csr_prepare");
     } else {
         TORCH_CHECK(rp.scalar_type() == torch::kInt32 && ci.scalar_type() == torch::kInt32,
                     "rowptr/col must be int64 or int32");
         blk->rowptr = rp;
         blk->colidx = ci;
-        blk->rowidx = torch::empty({blk->nnz}, i32);
-        ok(cgnn_csr_expand_rows(rows, blk->nnz, rp.data_ptr<int32_t>(),
-                                blk->nnz ? blk->rowidx.data_ptr<int32_t>() : nullptr, current_stream(rp)),
-           "csr_expand_rows");
     }
     if (value.has_value() && value->defined()) {
         TORCH_CHECK(value->numel() == blk->nnz, "value must have one entry per non-zero");
@@ -138,6 +172,7 @@ std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Ten
         Tensor lens = blk->rowptr.slice(0, 1, rows + 1) - blk->rowptr.slice(0, 0, rows);
         blk->max_row_nnz = lens.max().item<int32_t>();  // one host read per block, at build time
     }
+    if (with_row_lists) blk->list_rows();
     return blk;
 }
 
@@ -204,7 +239,7 @@ Tensor spmm_func(Tensor vlist, Tensor elist, Tensor value, Tensor mat, std::stri
     const int kernel = kernel_of_method(method);
     TORCH_CHECK(vlist.scalar_type() == torch::kInt64 && elist.scalar_type() == torch::kInt64,
                 "vlist and elist must be int64");
-    auto blk = make_csr(vlist, elist, value, vlist.size(-1) - 1, mat.size(0), mat.device(), 0);
+    auto blk = make_csr(vlist, elist, value, vlist.size(-1) - 1, mat.size(0), mat.device(), 0, c10::nullopt, false);
     return block_spmm(*blk, mat, optional_out, kernel);
 }
 
@@ -875,7 +910,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def_readonly("cols", &DeviceCsr::cols)
         .def_readonly("nnz", &DeviceCsr::nnz)
         .def_readonly("max_row_nnz", &DeviceCsr::max_row_nnz)
-        .def_readwrite("seg_nnz", &DeviceCsr::seg_nnz)
+        .def_property("seg_nnz", [](DeviceCsr &self) { return self.seg_nnz; },
+                      [](DeviceCsr &self, int32_t seg) {
+                          self.seg_nnz = seg;
+                          if (self.cut_rows.defined()) self.list_rows();  // the lists belong to a run length
+                      })
+        .def_readonly("cut_rows", &DeviceCsr::cut_rows)
+        .def_readonly("empty_rows", &DeviceCsr::empty_rows)
         .def_readwrite("stream_rows_over", &DeviceCsr::stream_rows_over)
         .def_readonly("rowptr", &DeviceCsr::rowptr)
         .def_readonly("colidx", &DeviceCsr::colidx)

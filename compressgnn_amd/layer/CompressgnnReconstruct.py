@@ -29,8 +29,12 @@ class _GatherBiasAct(torch.autograd.Function):
         ids = _dense(ids)
         lists = members_of(ids, reps.size(0))
         rows = _native.cluster_reconstruct(_dense(reps), ids, _dense(bias), relu, lists)
-        # the ReLU mask of the gradient is read off the rows that were produced
-        ctx.save_for_backward(ids, rows)
+        # the ReLU mask of the gradient is read off the rows that were produced; without a ReLU
+        # nothing of the [N, F] output is needed again, and nothing of it is kept
+        if relu:
+            ctx.save_for_backward(ids, rows)
+        else:
+            ctx.save_for_backward(ids)
         ctx.plan = (reps.size(0), relu, bias is not None, lists)
         return rows
 
@@ -38,8 +42,12 @@ class _GatherBiasAct(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, d_rows):
         clusters, relu, with_bias, lists = ctx.plan
-        ids, rows = ctx.saved_tensors
-        d_reps = _native.cluster_reconstruct_backward(_dense(d_rows), ids, rows, clusters, relu, lists)
+        d_rows = _dense(d_rows)
+        if relu:
+            ids, rows = ctx.saved_tensors
+        else:
+            (ids,), rows = ctx.saved_tensors, d_rows  # the operator wants a tensor of the shape; it is not read
+        d_reps = _native.cluster_reconstruct_backward(d_rows, ids, rows, clusters, relu, lists)
         return d_reps, None, (d_reps.sum(0) if with_bias else None), None
 
 

@@ -71,12 +71,31 @@ typedef struct cgnn_csr {
      * not kept in the L2 caches.  Pays only where the rows a hub gathers are not gathered again
      * soon by other rows; results are unchanged. */
     int32_t stream_rows_over;
+    /* NNZ schedule, optional (NULL = the fix-up pass looks at every run): the rows that the
+     * runs cut and the rows without entries, ascending, as numbers of stored rows.  With run
+     * length K = cgnn_spmm_run_length(A), row r is cut when rowptr[r+1] - rowptr[r] > K and
+     * (rowptr[r] / K + 1) * K < rowptr[r+1] (integer division: the row is longer than a run and a
+     * multiple of K lies strictly inside it; shorter rows are never cut).  Both lists
+     * follow from rowptr and K alone and must be exact when given (they are not checked);
+     * empty_rows may be NULL only if n_empty_rows is 0.  Results are unchanged. */
+    const int32_t *cut_rows;   /* [n_cut_rows] */
+    const int32_t *empty_rows; /* [n_empty_rows] */
+    int32_t n_cut_rows, n_empty_rows;
 } cgnn_csr;
 
 const char *cgnn_last_error(void);
 const char *cgnn_version(void);
 
 /* ------------------------------------------------------------------ SpMM ---- */
+
+/* The schedule CGNN_SPMM_AUTO stands for on a block of this shape that has rowidx (a block
+ * without rowidx always takes the ROW schedule under AUTO): lets a caller build rowidx, which the
+ * NNZ schedule alone reads, only for the blocks that will use it. */
+int cgnn_spmm_schedule(int64_t rows, int64_t nnz, int32_t max_row_nnz, int kernel);
+
+/* Non-zeros per run of the NNZ schedule for this block (seg_nnz, or the default, rounded up to
+ * what the kernels take). */
+int cgnn_spmm_run_length(const cgnn_csr *A);
 
 /* Bytes of scratch cgnn_spmm needs for this block, feature width and schedule
  * (the carry-out rows of the NNZ schedule).  0 for the ROW schedule. */

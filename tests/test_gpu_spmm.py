@@ -310,3 +310,43 @@ def test_csr_prepare_i64():
     assert np.array_equal(ci32.cpu().numpy(), elist.astype(np.int32))
     want = np.repeat(np.arange(rows), np.diff(vlist)).astype(np.int32)
     assert np.array_equal(ri.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("seg", [8, 32, 64])
+def test_fixup_over_row_lists_reads_only_fresh_carries(seg):
+    """A block built through the operator module knows which rows its runs cut (rows longer than a
+    run with a multiple of the run length inside) and looks only at those after the nnz kernel.
+    Short rows that merely contain such a multiple are not cut; the scratch is first filled with
+    NaN carries by a product over NaN input, so any carry slot that is read without having been
+    written in the same call shows up in the result."""
+    import compressgnn_runtime as rt
+    rng = np.random.default_rng(seg)
+    rows, cols, F = 3000, 800, 64
+    vlist, elist, value = random_csr(rng, rows, cols, 9.0, skew=True)
+    row_len = np.repeat(np.diff(vlist), np.diff(vlist))
+    value = (value * 0.3 / np.sqrt(np.maximum(row_len, 1))).astype(np.float32)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    A = rt.DeviceCsr(t(vlist), t(elist), t(value), rows, cols, torch.device(DEV), seg)
+    lens = np.diff(vlist)
+    K = (seg + 3) // 4 * 4
+    want_cut = np.nonzero((lens > K) & ((vlist[:-1] // K + 1) * K < vlist[1:]))[0]
+    assert np.array_equal(A.cut_rows.cpu().numpy(), want_cut.astype(np.int32))
+    assert np.array_equal(A.empty_rows.cpu().numpy(), np.nonzero(lens == 0)[0].astype(np.int32))
+    assert ((lens <= K) & ((vlist[:-1] // K + 1) * K < vlist[1:])).any()  # short rows over a multiple exist
+    want = oracle.spmm(vlist, elist, value, x)
+    X = t(x)
+    A.spmm(torch.full_like(X, float("nan")), None, "nnz_schedule")  # every carry slot that is written holds NaN now
+    got = A.spmm(X, None, "nnz_schedule")
+    assert_within(got.cpu().numpy(), want)
+    short = lens <= K
+    assert np.array_equal(got.cpu().numpy()[short], want[short])
+    out0 = rng.standard_normal((rows, F)).astype(np.float32)
+    A.spmm(torch.full_like(X, float("nan")), torch.zeros(rows, F, device=DEV), "nnz_schedule")
+    acc = t(out0.copy())
+    A.spmm(X, acc, "nnz_schedule")
+    assert_within(acc.cpu().numpy(), oracle.spmm(vlist, elist, value, x, out0.copy()))
+    assert np.array_equal(acc.cpu().numpy()[lens == 0], out0[lens == 0])
+    # the same block without the lists (the C ABI without cut_rows) gives the same bits
+    plain = abi.DeviceCsr.from_host(rows, cols, vlist, elist, value, DEV, seg_nnz=seg)
+    assert torch.equal(abi.spmm(plain, X, None, False, abi.SPMM_NNZ), got)
