@@ -573,6 +573,42 @@ def main():
         if not args.skip_cpu:
             cpu_cluster_baseline(xc, planes, detail)
 
+    # neighbour sampling over the compressed C1 graph: two layers of 10 in-neighbours for every
+    # eighth vertex (the sampler's own copies of the int64 blocks; two scalar reads per layer)
+    try:
+        import compressgnn_sample as sampler
+        seeds = torch.arange(0, C1_VERTICES, 8, device=dev)
+        fan = [10, 10]
+        res = sampler.sample_compress_graph(graph, seeds, fan, seed=1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps_s = 5
+        for k in range(reps_s):
+            res = sampler.sample_compress_graph(graph, seeds, fan, seed=k)
+        torch.cuda.synchronize()
+        s_ms = (time.perf_counter() - t0) / reps_s * 1e3
+        detail["neighbor_sampler_C1"] = dict(seeds=int(seeds.numel()), fanout=fan, ms=s_ms, sampled_vertices=int(res[0].numel()),
+                                             sampled_edges=int(res[1].numel()),
+                                             edges_per_second=int(res[1].numel()) / (s_ms * 1e-3))
+        if not args.skip_cpu:
+            # the reference's own CPU sampler on the same graph and seeds (oracle/_ref, this leg only)
+            try:
+                sys.path.insert(0, os.path.join(ROOT, "oracle", "_ref"))
+                import compressgnn_sample_ref as cpu_sampler
+                held = [t.cpu() if torch.is_tensor(t) else [u.cpu() for u in t] for t in graph._sampler_blocks[1]]
+                torch.manual_seed(0)
+                t0 = time.perf_counter()
+                cpu_res = cpu_sampler.neighbor_sample_cg_sim(*held, seeds.cpu(), fan)
+                detail["neighbor_sampler_C1"]["cpu_reference_ms"] = (time.perf_counter() - t0) * 1e3
+                detail["neighbor_sampler_C1"]["cpu_reference_edges"] = int(cpu_res[1].numel())
+            except Exception as exc:
+                detail["neighbor_sampler_C1"]["cpu_reference_ms"] = None
+                log("[bench] CPU sampler not timed: %r" % (exc,))
+        graph._sampler_blocks = None
+        del res, seeds
+    except Exception as exc:
+        detail["neighbor_sampler_C1"] = dict(error="%s: %s" % (type(exc).__name__, exc))
+
     if not args.skip_c4:
         # the large end-to-end configuration, after everything of C1 and C3 has left the device
         del x, g, out, gx, ref_out, plan, graph, data
