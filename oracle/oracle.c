@@ -14,6 +14,9 @@
  *                        (tests/test_transformation.py:16-20), golden (index, active) of
  *                        the compiled cluster_forward on inputs whose projections are
  *                        exactly representable, known answers count == [0, 513]
+ *   - the sampler (oracle_sample.c) : the compiled reference's own outputs, its draws replayed
+ *                        from torch's CPU generator; its counter-based generator is this
+ *                        build's definition and "parity unpinned" (see that file's header)
  *   - cluster_mean_*, reconstruct_* : index_add / index_select closed forms of
  *                        layer/CompressgnnCluster.py:16-25 and
  *                        layer/CompressgnnReconstruct.py:39-42, float64 finite differences

@@ -52,4 +52,7 @@ def assert_no_less_accurate(got, sequential, truth, factor=2.0):
         "kernel is %.3e from the float64 result, the sequential fp32 sum %.3e" % (e_got.max(), e_seq.max())
     assert e_got.mean() <= factor * e_seq.mean() + floor, \
         "mean error: kernel %.3e, sequential fp32 sum %.3e" % (e_got.mean(), e_seq.mean())
+    # one line for the record (shown with pytest -s)
+    print("accuracy vs float64: kernel max %.3e mean %.3e | sequential fp32 max %.3e mean %.3e" % (
+        e_got.max(), e_got.mean(), e_seq.max(), e_seq.mean()))
     return float(e_got.max()), float(e_seq.max())
