@@ -11,9 +11,9 @@
  * that very generator (the sampling loop then reproduces the compiled reference exactly,
  * which is how this file is pinned: tests/test_oracle_sample.py against oracle/_ref and the
  * golden vectors written from it), or from the counter-based generator the HIP sampler uses
- * (oracle_counter_draw below, this build's own definition: the reference has no device
- * sampler, so the stream of random numbers on the GPU has nothing to be compared with; what
- * is compared is everything that follows from a given stream).
+ * (oracle_counter_draw below: PARITY UNPINNED -- it is this build's own definition; the
+ * reference has no device sampler, so the stream of random numbers on the GPU has nothing to
+ * be compared with; what is compared is everything that follows from a given stream).
  * Further pins: the expansion invariant (the neighbours enumerated by get_neighbor over all
  * indices, and the full list, are the expanded in-list of the vertex) on graphs whose rule
  * hierarchy the reference's degree computation covers.
