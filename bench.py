@@ -253,6 +253,13 @@ def bench_cluster(torch, steps, detail):
     t_recon, out = timed(lambda: rt.cluster_reconstruct(hidden, ids, bias, True, members))
     grad_out = torch.randn(N, Fo, device=dev, generator=gen)
     t_recon_bwd, hidden_grad = timed(lambda: rt.cluster_reconstruct_backward(grad_out, ids, out, groups, True, members))
+    # the pair the layer runs: the ReLU mask travels as one bit per element, written by the forward kernel
+    t_recon_s, (out_s, signs) = timed(lambda: rt.cluster_reconstruct_signs(hidden, ids, bias, members))
+    t_recon_bwd_s, hidden_grad_s = timed(lambda: rt.cluster_reconstruct_backward_signs(grad_out, ids, signs, groups, members))
+    if not (torch.equal(out_s, out) and torch.equal(hidden_grad_s, hidden_grad)):
+        raise RuntimeError("the sign-bit form of reconstruct disagrees with the form that keeps the rows")
+    W = signs.size(1)
+    del out_s, hidden_grad_s
     t_linear_bwd, reps_grad = timed(lambda: hidden_grad @ weight)
     t_mean_bwd, dx = timed(lambda: rt.cluster_mean_backward(reps_grad, ids, counts, members))
     gb = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
@@ -263,18 +270,27 @@ def bench_cluster(torch, steps, detail):
         "reconstruct": dict(ms=t_recon, bytes=4 * C * Fo + 8 * N + 4 * Fo + 4 * N * Fo),
         "reconstruct_backward": dict(ms=t_recon_bwd, bytes=2 * 4 * N * Fo + 8 * N + 4 * C * Fo),
         "mean_backward": dict(ms=t_mean_bwd, bytes=4 * C * F + 8 * N + 4 * N * F),
+        "reconstruct_signs": dict(ms=t_recon_s, bytes=4 * C * Fo + 8 * N + 4 * Fo + 4 * N * Fo + 4 * N * W),
+        "reconstruct_backward_signs": dict(ms=t_recon_bwd_s, bytes=4 * N * Fo + 4 * N * W + 8 * N + 4 * C * Fo),
     }
     for k, v in ops.items():
         v["GBps"] = gb(v["bytes"], v["ms"])
         v["frac_of_hbm_peak"] = v["GBps"] / HBM_PEAK_GBPS
-    reuse = t_mean + t_linear + t_recon + t_recon_bwd + t_linear_bwd + t_mean_bwd
+    # an epoch of the layers (Compressgnn_Cluster -> Linear -> Compressgnn_Reconstruct with ReLU): the sign-bit pair;
+    # beside it the same chain through the operators with the reference's signatures, which read the rows back
+    rest = t_mean + t_linear + t_linear_bwd + t_mean_bwd
+    reuse = rest + t_recon_s + t_recon_bwd_s
     refresh = reuse + t_assign
+    reuse_rows = rest + t_recon + t_recon_bwd
     detail["cluster_reconstruct_C3"] = dict(
         nodes=N, in_features=F, bits=C3_H, out_features=Fo, active_clusters=int(active), ops=ops,
         linear_ms=t_linear, linear_backward_ms=t_linear_bwd,
         fwd_bwd_ms_refresh_epoch=refresh, fwd_bwd_ms_reuse_epoch=reuse,
         fwd_bwd_ms_per_epoch_refresh_interval_1=refresh,
-        fwd_bwd_ms_per_epoch_refresh_interval_5=(refresh + 4 * reuse) / 5)
+        fwd_bwd_ms_per_epoch_refresh_interval_5=(refresh + 4 * reuse) / 5,
+        reference_signature_operators=dict(
+            fwd_bwd_ms_per_epoch_refresh_interval_1=reuse_rows + t_assign,
+            fwd_bwd_ms_per_epoch_refresh_interval_5=(reuse_rows + t_assign + 4 * reuse_rows) / 5))
     log("[bench] C3 cluster+reconstruct: " + ", ".join("%s %.3f ms (%.0f GB/s)" % (k, v["ms"], v["GBps"])
                                                         for k, v in ops.items()))
     return x, planes

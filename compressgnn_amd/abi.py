@@ -26,7 +26,8 @@ EXPORTS = [
     "cgnn_lsh_group_workspace_bytes", "cgnn_lsh_group",
     "cgnn_cluster_members_workspace_bytes", "cgnn_cluster_members",
     "cgnn_cluster_mean_workspace_bytes", "cgnn_cluster_mean", "cgnn_cluster_mean_backward",
-    "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_copy_bytes", "cgnn_read_bytes", "cgnn_fill_bytes",
+    "cgnn_reconstruct", "cgnn_reconstruct_backward", "cgnn_sign_words", "cgnn_reconstruct_signs",
+    "cgnn_reconstruct_backward_signs", "cgnn_copy_bytes", "cgnn_read_bytes", "cgnn_fill_bytes",
     "cgnn_exclusive_sum_workspace_bytes", "cgnn_exclusive_sum_i32", "cgnn_sample_count", "cgnn_sample_fill",
     "cgnn_sample_relabel_begin", "cgnn_sample_relabel_workspace_bytes", "cgnn_sample_relabel",
 ]
@@ -313,6 +314,35 @@ def reconstruct(reps, ids, bias=None, relu=False, members=None):
                                  ptr(bad), stream_of(reps)))
     _check_id_flag(bad, "reconstruct", reps.shape[0])
     return out
+
+
+def reconstruct_signs(reps, ids, bias=None, members=None):
+    """(rows with ReLU, int32 [N, ceil(F / 32)] sign bits)"""
+    N = ids.numel()
+    F = reps.shape[1]
+    L = lib()
+    L.cgnn_sign_words.restype = ctypes.c_int64
+    out = torch.empty((N, F), dtype=reps.dtype, device=reps.device)
+    signs = torch.empty((N, L.cgnn_sign_words(i64(F))), dtype=torch.int32, device=reps.device)
+    perm = None if members is None else members[1]
+    bad = _id_flag(reps.device)
+    check(L.cgnn_reconstruct_signs(i64(N), i64(F), i64(reps.shape[0]), dtype_code(reps.dtype), ptr(reps), ptr(ids),
+                                   ptr(perm), ptr(bias), ptr(out), ptr(signs), ptr(bad), stream_of(reps)))
+    _check_id_flag(bad, "reconstruct_signs", reps.shape[0])
+    return out, signs
+
+
+def reconstruct_backward_signs(grad, signs, members, groups, max_members=0):
+    offsets, perm, sorted_id = members[:3]
+    N, F = grad.shape
+    L = lib()
+    reps_grad = torch.empty((groups, F), dtype=grad.dtype, device=grad.device)
+    need = L.cgnn_cluster_mean_workspace_bytes(i64(N), i64(F), i64(groups), dtype_code(grad.dtype))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=grad.device)
+    check(L.cgnn_reconstruct_backward_signs(i64(N), i64(F), i64(groups), i64(max_members), dtype_code(grad.dtype),
+                                            ptr(grad), ptr(signs), ptr(offsets), ptr(perm), ptr(sorted_id),
+                                            ptr(reps_grad), ptr(ws), ctypes.c_size_t(need), stream_of(grad)))
+    return reps_grad
 
 
 def reconstruct_backward(grad, output, members, groups, relu=False, max_members=0):

@@ -9,7 +9,7 @@
 namespace cgnn {
 
 int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, void *Y, int64_t F,
-                 bool relu_mask, void *ws, size_t ws_bytes, hipStream_t stream);
+                 int mask, void *ws, size_t ws_bytes, hipStream_t stream);
 
 namespace {
 
@@ -749,8 +749,10 @@ struct GatherArgs {
     const T *__restrict__ bias;
     T *__restrict__ out;             // [N x F]
     int32_t *bad_id;                 // set to 1 when an id lies outside [0, groups), or NULL
+    uint32_t *signs;                 // reconstruct: bit f % 32 of word [i, f / 32] = !(out[i, f] <= 0), or NULL
     int64_t N, F, groups;
     int32_t relu;
+    int32_t sign_words;              // words per row of signs: ceil(F / 32)
 };
 
 // Output rows are written once and not read again here: streaming stores.
@@ -794,30 +796,54 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
 #pragma unroll
         for (int r = 0; r < kGatherRows; ++r) denom[r] = (T)max(a.counts[g[r]], 1);
     }
-    for (int64_t f = (int64_t)lane * VEC; f < a.F; f += (int64_t)LPR * VEC) {
+    // the lanes of a row walk the features together (a lane past the end of the row idles), so that
+    // lanes can exchange sign bits below
+    for (int64_t fb = 0; fb < a.F; fb += (int64_t)LPR * VEC) {
+        const int64_t f = fb + (int64_t)lane * VEC;
+        const bool on = f < a.F;
         LPack<T, VEC> x[kGatherRows];
+        uint32_t bits[kGatherRows];
 #pragma unroll
-        for (int r = 0; r < kGatherRows; ++r)
-            x[r] = *reinterpret_cast<const LPack<T, VEC> *>(a.src + g[r] * a.F + f);
-        LPack<T, VEC> b;
-        if constexpr (OP == GATHER_RECONSTRUCT) {
-            if (a.bias) b = *reinterpret_cast<const LPack<T, VEC> *>(a.bias + f);
-        }
+        for (int r = 0; r < kGatherRows; ++r) bits[r] = 0;
+        if (on) {
 #pragma unroll
-        for (int r = 0; r < kGatherRows; ++r) {
-            if (first + r >= a.N) break;
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                T v = x[r].v[i];
-                if constexpr (OP == GATHER_MEAN_GRAD) {
-                    v = v / denom[r];
-                } else {
-                    if (a.bias) v = v + b.v[i];
-                    v = (a.relu && v < T(0)) ? T(0) : v;
-                }
-                x[r].v[i] = v;
+            for (int r = 0; r < kGatherRows; ++r)
+                x[r] = *reinterpret_cast<const LPack<T, VEC> *>(a.src + g[r] * a.F + f);
+            LPack<T, VEC> b;
+            if constexpr (OP == GATHER_RECONSTRUCT) {
+                if (a.bias) b = *reinterpret_cast<const LPack<T, VEC> *>(a.bias + f);
             }
-            store_stream<T, VEC>(a.out + row[r] * a.F + f, x[r]);
+#pragma unroll
+            for (int r = 0; r < kGatherRows; ++r) {
+                if (first + r >= a.N) break;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    T v = x[r].v[i];
+                    if constexpr (OP == GATHER_MEAN_GRAD) {
+                        v = v / denom[r];
+                    } else {
+                        if (a.bias) v = v + b.v[i];
+                        v = (a.relu && v < T(0)) ? T(0) : v;
+                        bits[r] |= (v <= T(0) ? 0u : 1u) << i;
+                    }
+                    x[r].v[i] = v;
+                }
+                store_stream<T, VEC>(a.out + row[r] * a.F + f, x[r]);
+            }
+        }
+        if constexpr (OP == GATHER_RECONSTRUCT) {
+            if (a.signs != nullptr) {
+                // VEC divides 32: the lanes whose bits share a word are R neighbours within the row's lanes
+                constexpr int R = LPR < 32 / VEC ? LPR : 32 / VEC;
+#pragma unroll
+                for (int r = 0; r < kGatherRows; ++r) {
+                    if (first + r >= a.N) break;  // the same for all lanes of the row
+                    uint32_t w = bits[r] << (f & 31);
+#pragma unroll
+                    for (int d = 1; d < R; d <<= 1) w |= __shfl_xor(w, d);
+                    if (on && lane % R == 0) a.signs[row[r] * a.sign_words + (f >> 5)] = w;
+                }
+            }
         }
     }
 }
@@ -1037,7 +1063,7 @@ extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int64_t m
     CGNN_REQUIRE(offsets && counts && reps, "cgnn_cluster_mean: null array");
     CGNN_REQUIRE(N == 0 || (X && perm && sorted_id), "cgnn_cluster_mean: null array");
     cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id, max_members);
-    int rc = spmm_members(&A, dtype, X, nullptr, reps, F, false, workspace, workspace_bytes, stream);
+    int rc = spmm_members(&A, dtype, X, nullptr, reps, F, 0, workspace, workspace_bytes, stream);
     if (rc != CGNN_OK) return rc;
     if (dtype == CGNN_F32) return divide_counts<float>(reps, counts, groups, F, stream);
     return divide_counts<double>(reps, counts, groups, F, stream);
@@ -1046,8 +1072,10 @@ extern "C" int cgnn_cluster_mean(int64_t N, int64_t F, int64_t groups, int64_t m
 template <typename T, int OP>
 static int gather_typed(int64_t N, int64_t F, int64_t groups, const void *src, const int64_t *ids,
                         const int32_t *counts, const int32_t *perm, const void *bias, int relu, void *out,
-                        int32_t *bad_id, hipStream_t stream) {
+                        int32_t *bad_id, hipStream_t stream, uint32_t *signs = nullptr) {
     GatherArgs<T> a{};
+    a.signs = signs;
+    a.sign_words = (int32_t)ceil_div(F, 32);
     a.src = static_cast<const T *>(src);
     a.ids = ids;
     a.counts = counts;
@@ -1104,8 +1132,37 @@ extern "C" int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, i
     CGNN_REQUIRE(N == 0 || (grad && perm && sorted_id), "cgnn_reconstruct_backward: null array");
     CGNN_REQUIRE(!relu || N == 0 || output, "cgnn_reconstruct_backward: relu needs the saved output");
     cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id, max_members);
-    return spmm_members(&A, dtype, grad, output, reps_grad, F, relu != 0, workspace, workspace_bytes,
+    return spmm_members(&A, dtype, grad, output, reps_grad, F, relu != 0 ? 1 : 0, workspace, workspace_bytes,
                         stream);
+}
+
+extern "C" int64_t cgnn_sign_words(int64_t F) { return F <= 0 ? 0 : (F + 31) / 32; }
+
+extern "C" int cgnn_reconstruct_signs(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
+                                      const int64_t *ids, const int32_t *perm, const void *bias, void *out,
+                                      uint32_t *signs, int32_t *bad_id, cgnn_stream_t stream) {
+    CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 0, "cgnn_reconstruct_signs: bad size");
+    CGNN_REQUIRE(N == 0 || F == 0 || groups >= 1, "cgnn_reconstruct_signs: rows to reconstruct but no representatives");
+    if (N == 0 || F == 0) return CGNN_OK;
+    CGNN_REQUIRE(reps && ids && out && signs, "cgnn_reconstruct_signs: null array");
+    if (dtype == CGNN_F32)
+        return gather_typed<float, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, 1, out, bad_id, stream, signs);
+    if (dtype == CGNN_F64)
+        return gather_typed<double, GATHER_RECONSTRUCT>(N, F, groups, reps, ids, nullptr, perm, bias, 1, out, bad_id, stream, signs);
+    return fail(CGNN_EUNSUPPORTED, "cgnn_reconstruct_signs: dtype must be f32 or f64");
+}
+
+extern "C" int cgnn_reconstruct_backward_signs(int64_t N, int64_t F, int64_t groups, int64_t max_members, int dtype,
+                                               const void *grad, const uint32_t *signs, const int32_t *offsets,
+                                               const int32_t *perm, const int32_t *sorted_id, void *reps_grad,
+                                               void *workspace, size_t workspace_bytes, cgnn_stream_t stream) {
+    CGNN_REQUIRE(N >= 0 && F >= 0 && groups >= 0, "cgnn_reconstruct_backward_signs: bad size");
+    CGNN_REQUIRE(dtype == CGNN_F32 || dtype == CGNN_F64, "cgnn_reconstruct_backward_signs: dtype must be f32 or f64");
+    if (F == 0 || groups == 0) return CGNN_OK;
+    CGNN_REQUIRE(offsets && reps_grad, "cgnn_reconstruct_backward_signs: null array");
+    CGNN_REQUIRE(N == 0 || (grad && perm && sorted_id && signs), "cgnn_reconstruct_backward_signs: null array");
+    cgnn_csr A = members_csr(N, groups, offsets, perm, sorted_id, max_members);
+    return spmm_members(&A, dtype, grad, signs, reps_grad, F, 2, workspace, workspace_bytes, stream);
 }
 
 extern "C" int cgnn_read_bytes(const void *src, size_t n, void *sink, cgnn_stream_t stream) {

@@ -53,7 +53,7 @@ constexpr int kRowUnroll = 4;     // same for the row schedule (8: 9 % slower on
 constexpr int kXcds = 8;          // accelerator dies of an MI355X, each with its own L2
 constexpr int kDefaultSeg = 64;   // non-zeros per lane group in the nnz schedule
 
-enum { MODE_VAL = 0, MODE_UNIT = 1, MODE_RELU_MASK = 2, MODE_DUAL = 3 };
+enum { MODE_VAL = 0, MODE_UNIT = 1, MODE_RELU_MASK = 2, MODE_DUAL = 3, MODE_SIGN_MASK = 4 };
 
 template <typename T, int VEC>
 struct alignas(sizeof(T) * VEC) Pack {
@@ -70,6 +70,8 @@ struct SpmmArgs {
     const T *X;   // gathered matrix (may alias Y)
     const T *X1;  // MODE_DUAL: source of the columns >= split
     const T *M;   // MODE_RELU_MASK: rows of X are zeroed where M <= 0
+    const uint32_t *signs;  // MODE_SIGN_MASK: the same with one bit per element (set: keep), sign_words words per row
+    int32_t sign_words;
     T *Y;
     int32_t *carry_row;  // [nseg] row a run carries into, or -1
     T *carry;            // [nseg x F]
@@ -225,7 +227,7 @@ __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_
 }
 
 // Gather one feature tile of column c (source chosen by `src` in MODE_DUAL, masked by
-// M in MODE_RELU_MASK).
+// M in MODE_RELU_MASK and by the bits of `signs` in MODE_SIGN_MASK).
 template <typename T, int VEC, int MODE>
 __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int src, int64_t foff, bool stream = false) {
     Pack<T, VEC> x;
@@ -244,8 +246,16 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
     const int64_t off = (int64_t)c * (int32_t)a.F + foff;  // F < 2^31: one 32 x 32 -> 64 bit multiply
     // rows that are gathered once (member lists; masks exist for those only) are not kept in the caches
     // (`stream`: the same for the runs of hub rows of a graph block when the block asks for it; uniform over the wave)
-    if (MODE == MODE_RELU_MASK || (MODE == MODE_UNIT && a.read_once) || stream) x = load_pack_stream<T, VEC>(base + off);
-    else x = load_pack<T, VEC>(base + off);
+    if (MODE == MODE_RELU_MASK || MODE == MODE_SIGN_MASK || (MODE == MODE_UNIT && a.read_once) || stream)
+        x = load_pack_stream<T, VEC>(base + off);
+    else
+        x = load_pack<T, VEC>(base + off);
+    if constexpr (MODE == MODE_SIGN_MASK) {
+        // VEC divides 32, so the bits of one pack lie in one word
+        const uint32_t bits = a.signs[(int64_t)c * a.sign_words + (foff >> 5)] >> (foff & 31);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = ((bits >> i) & 1u) ? x.v[i] : T(0);
+    }
     if constexpr (MODE == MODE_RELU_MASK) {
         Pack<T, VEC> m = load_pack_stream<T, VEC>(a.M + off);
 #pragma unroll
@@ -929,6 +939,8 @@ int launch_shape(int kind, int mode, const SpmmArgs<T> &args, int64_t items, int
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_UNIT>), grid, block, 0, stream, a);
             else if (mode == MODE_DUAL)
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_DUAL>), grid, block, 0, stream, a);
+            else if (mode == MODE_SIGN_MASK)
+                hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_SIGN_MASK>), grid, block, 0, stream, a);
             else
                 hipLaunchKernelGGL((spmm_nnz_kernel<T, VEC, LPR, TILES, MODE_RELU_MASK>), grid, block, 0, stream, a);
             break;
@@ -1082,10 +1094,17 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     if (A->rows == 0 || F == 0) return CGNN_OK;
     if (mode != MODE_DUAL) split = INT32_MAX;  // every column comes from X
     SpmmArgs<T> a = make_args<T>(A, X, X1, split, M, Y, F, accumulate);
-    a.read_once = mode == MODE_UNIT || mode == MODE_RELU_MASK;  // asked for by name: the cluster reductions
+    const bool masked = mode == MODE_RELU_MASK || mode == MODE_SIGN_MASK;
+    a.read_once = mode == MODE_UNIT || masked;  // asked for by name: the cluster reductions
+    if (mode == MODE_SIGN_MASK) {  // M holds bits, not rows
+        a.signs = static_cast<const uint32_t *>(M);
+        a.sign_words = (int32_t)ceil_div(F, 32);
+        a.M = nullptr;
+        M = nullptr;
+    }
     a.stream_over = A->stream_rows_over > 0 ? A->stream_rows_over : 0;
     kernel = resolve_kernel(A, kernel);
-    if (mode == MODE_RELU_MASK) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
+    if (masked) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
     if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;
     if (mode == MODE_DUAL && A->nnz > 0 && A->val == nullptr)
         return fail(CGNN_EINVAL, "spmm: the two-source product needs stored values");
@@ -1178,10 +1197,11 @@ unsigned grid_for(int64_t n) {
 
 }  // namespace
 
-// Entry used by the cluster reductions (unit values, optional ReLU mask).
+// Entry used by the cluster reductions (unit values; mask: 0 none, 1 the rows of M, where M <= 0 drops
+// the element, 2 M holds ceil(F / 32) words of bits per row, where a clear bit drops it).
 int spmm_members(const cgnn_csr *A, int dtype, const void *X, const void *M, void *Y, int64_t F,
-                 bool relu_mask, void *ws, size_t ws_bytes, hipStream_t stream) {
-    const int mode = relu_mask ? MODE_RELU_MASK : MODE_UNIT;
+                 int mask, void *ws, size_t ws_bytes, hipStream_t stream) {
+    const int mode = mask == 2 ? MODE_SIGN_MASK : (mask == 1 ? MODE_RELU_MASK : MODE_UNIT);
     if (dtype == CGNN_F32)
         return spmm_typed<float>(A, X, nullptr, 0, M, Y, F, 0, CGNN_SPMM_NNZ, mode, ws, ws_bytes, stream);
     if (dtype == CGNN_F64)

@@ -682,6 +682,60 @@ Tensor cluster_reconstruct_backward(Tensor grad, Tensor index, Tensor output, in
     return out;
 }
 
+// The ReLU form of cluster_reconstruct that also returns the sign of every output element as one
+// bit: (rows [N, F], signs int32 [N, ceil(F / 32)]).  A layer keeps the signs for its backward pass
+// instead of the rows (the reference keeps the rows: layer/CompressgnnReconstruct.py:16-22).
+std::tuple<Tensor, Tensor> cluster_reconstruct_signs(Tensor reps, Tensor index, c10::optional<Tensor> bias,
+                                                     c10::optional<std::vector<Tensor>> members) {
+    const char *op = "cluster_reconstruct_signs";
+    expect(op, reps, {{Role::Features, "representatives", &reps}, {Role::Ids, "index", &index}});
+    if (bias.has_value()) {
+        expect(op, reps, {{Role::Bias, "bias", &*bias}});
+        TORCH_CHECK(bias->numel() == reps.size(1), op, ": a bias of ", bias->numel(), " entries for rows of ", reps.size(1));
+    }
+    TORCH_CHECK(index.numel() == 0 || reps.size(0) > 0, op, ": rows to reconstruct but no representatives");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(reps.device());
+    const int64_t N = index.numel(), F = reps.size(1);
+    Tensor out = torch::empty({N, F}, reps.options());
+    Tensor signs = torch::empty({N, cgnn_sign_words(F)}, reps.options().dtype(torch::kInt32));
+    if (out.numel() == 0) return {out, signs};
+    const int32_t *perm = production_order(op, members, index);
+    c10::optional<IdFlag> bad;
+    if (perm == nullptr) bad.emplace(index);
+    ok(cgnn_reconstruct_signs(N, F, reps.size(0), dtype_code(reps), reps.data_ptr(), index.data_ptr<int64_t>(), perm,
+                              bias.has_value() ? bias->data_ptr() : nullptr, out.data_ptr(),
+                              reinterpret_cast<uint32_t *>(signs.data_ptr<int32_t>()), bad ? bad->ptr() : nullptr,
+                              current_stream(reps)),
+       op);
+    if (bad) bad->raise(op, reps.size(0));
+    return {out, signs};
+}
+
+// cluster_reconstruct_backward with relu = true, the mask taken from the signs above.
+Tensor cluster_reconstruct_backward_signs(Tensor grad, Tensor index, Tensor signs, int64_t groups,
+                                          c10::optional<std::vector<Tensor>> members) {
+    const char *op = "cluster_reconstruct_backward_signs";
+    expect(op, grad, {{Role::Features, "grad", &grad}, {Role::Ids, "index", &index}});
+    TORCH_CHECK(groups >= 0, op, ": groups = ", groups);
+    TORCH_CHECK(index.numel() == grad.size(0), op, ": ", grad.size(0), " rows but ", index.numel(), " cluster ids");
+    const int64_t N = grad.size(0), F = grad.size(1);
+    TORCH_CHECK(signs.device() == grad.device() && signs.scalar_type() == torch::kInt32 && signs.is_contiguous() &&
+                    signs.dim() == 2 && signs.size(0) == N && signs.size(1) == cgnn_sign_words(F),
+                op, ": signs must be a contiguous int32 tensor [", N, ", ", cgnn_sign_words(F), "] on the device of grad");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
+    if (grad.numel() == 0 || groups == 0) return torch::zeros({groups, F}, grad.options());
+    auto m = members_or_build(op, members, index, groups);
+    Tensor out = torch::empty({groups, F}, grad.options());
+    const size_t bytes = cgnn_cluster_mean_workspace_bytes(N, F, groups, dtype_code(grad));
+    Tensor ws = torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, grad.options().dtype(torch::kUInt8));
+    ok(cgnn_reconstruct_backward_signs(N, F, groups, largest_group(m), dtype_code(grad), grad.data_ptr(),
+                                       reinterpret_cast<const uint32_t *>(signs.data_ptr<int32_t>()),
+                                       m[0].data_ptr<int32_t>(), m[1].data_ptr<int32_t>(), m[2].data_ptr<int32_t>(),
+                                       out.data_ptr(), ws.data_ptr(), bytes, current_stream(grad)),
+       op);
+    return out;
+}
+
 // (colptr, row, value) of a block held as int64 tensors on a GPU: the CSR of its transpose,
 // in the order SparseTensor.csc() gives.  The one host read (a flag for columns out of
 // range) comes after the last kernel.
@@ -895,6 +949,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("colptr"), py::arg("row"), py::arg("input_node"), py::arg("num_neighbors"), py::arg("seed") = 0);
     // additions of this build
     m.def("cluster_members", &cluster_members, "member lists (offsets, perm, sorted_id) of the clusters");
+    m.def("cluster_reconstruct_signs", &cluster_reconstruct_signs,
+          "cluster_reconstruct with ReLU -> (rows, one sign bit per element)", py::arg("reps"), py::arg("index"),
+          py::arg("bias"), py::arg("members") = py::none());
+    m.def("cluster_reconstruct_backward_signs", &cluster_reconstruct_backward_signs,
+          "cluster_reconstruct_backward with ReLU, masked by the sign bits", py::arg("grad"), py::arg("index"),
+          py::arg("signs"), py::arg("groups"), py::arg("members") = py::none());
     m.def("csr_transpose", &csr_transpose, "CSR -> CSC of an int64 block on the GPU, SparseTensor.csc() order",
           py::arg("rowptr"), py::arg("col"), py::arg("value"), py::arg("cols"));
     m.def("version", []() { return std::string(cgnn_version()); });

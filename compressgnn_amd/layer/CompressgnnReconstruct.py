@@ -28,12 +28,14 @@ class _GatherBiasAct(torch.autograd.Function):
     def forward(ctx, reps, ids, bias, relu):
         ids = _dense(ids)
         lists = members_of(ids, reps.size(0))
-        rows = _native.cluster_reconstruct(_dense(reps), ids, _dense(bias), relu, lists)
-        # the ReLU mask of the gradient is read off the rows that were produced; without a ReLU
-        # nothing of the [N, F] output is needed again, and nothing of it is kept
+        # The ReLU mask of the gradient is kept as one bit per element, written by the kernel that
+        # produces the rows (the reference keeps the rows themselves, :16-22); without a ReLU
+        # nothing of the [N, F] output is needed again.  Either way none of it is kept.
         if relu:
-            ctx.save_for_backward(ids, rows)
+            rows, signs = _native.cluster_reconstruct_signs(_dense(reps), ids, _dense(bias), lists)
+            ctx.save_for_backward(ids, signs)
         else:
+            rows = _native.cluster_reconstruct(_dense(reps), ids, _dense(bias), False, lists)
             ctx.save_for_backward(ids)
         ctx.plan = (reps.size(0), relu, bias is not None, lists)
         return rows
@@ -44,10 +46,12 @@ class _GatherBiasAct(torch.autograd.Function):
         clusters, relu, with_bias, lists = ctx.plan
         d_rows = _dense(d_rows)
         if relu:
-            ids, rows = ctx.saved_tensors
+            ids, signs = ctx.saved_tensors
+            d_reps = _native.cluster_reconstruct_backward_signs(d_rows, ids, signs, clusters, lists)
         else:
-            (ids,), rows = ctx.saved_tensors, d_rows  # the operator wants a tensor of the shape; it is not read
-        d_reps = _native.cluster_reconstruct_backward(d_rows, ids, rows, clusters, relu, lists)
+            (ids,) = ctx.saved_tensors
+            # the operator wants a tensor of the shape of the output; without a ReLU it is not read
+            d_reps = _native.cluster_reconstruct_backward(d_rows, ids, d_rows, clusters, False, lists)
         return d_reps, None, (d_reps.sum(0) if with_bias else None), None
 
 

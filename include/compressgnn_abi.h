@@ -273,6 +273,22 @@ int cgnn_reconstruct_backward(int64_t N, int64_t F, int64_t groups, int64_t max_
                               const int32_t *sorted_id, int relu, void *reps_grad,
                               void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
 
+/* The ReLU mask as one bit per element.  cgnn_reconstruct_signs is cgnn_reconstruct with relu = 1
+ * that also writes signs[i * W + f / 32], W = cgnn_sign_words(F) = ceil(F / 32): bit f % 32 is set
+ * unless out[i,f] <= 0 (bits past F are clear).  cgnn_reconstruct_backward_signs is
+ * cgnn_reconstruct_backward with relu = 1 that drops grad[i,f] where the bit is clear, so it reads
+ * N * W words in place of the N x F saved output and gives the same reps_grad bit for bit.
+ * No counterpart in the reference, whose layer keeps the whole output for its backward pass
+ * (layer/CompressgnnReconstruct.py:16-26, cluster_kernel.cu:196-208). */
+int64_t cgnn_sign_words(int64_t F);
+int cgnn_reconstruct_signs(int64_t N, int64_t F, int64_t groups, int dtype, const void *reps,
+                           const int64_t *ids, const int32_t *perm, const void *bias, void *out,
+                           uint32_t *signs, int32_t *bad_id, cgnn_stream_t stream);
+int cgnn_reconstruct_backward_signs(int64_t N, int64_t F, int64_t groups, int64_t max_members, int dtype,
+                                    const void *grad, const uint32_t *signs, const int32_t *offsets,
+                                    const int32_t *perm, const int32_t *sorted_id, void *reps_grad,
+                                    void *workspace, size_t workspace_bytes, cgnn_stream_t stream);
+
 /* ---------------------------------------- neighbour sampling on a compressed graph -- */
 
 /* The work of the reference's CPU module compressgnn_sample

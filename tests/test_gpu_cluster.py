@@ -22,6 +22,18 @@ def _t(a):
     return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
 
 
+def pack_signs(out):
+    """The sign words of cgnn_reconstruct_signs from the rows: bit f % 32 of word f // 32 is set
+    unless out[i, f] <= 0 (so a NaN keeps its bit, as it keeps its gradient in the reference's mask,
+    cluster_kernel.cu:98-108); bits past the width are clear."""
+    n, width = out.shape
+    words = (width + 31) // 32
+    bits = np.zeros((n, words * 32), dtype=np.uint64)
+    bits[:, :width] = ~(out <= 0)
+    packed = (bits.reshape(n, words, 32) << np.arange(32, dtype=np.uint64)).sum(axis=2)
+    return packed.astype(np.uint32).view(np.int32)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("width", [0, 1, 31, 33, 100, 128, 602])
 @pytest.mark.parametrize("n,bits", [(1, 0), (67, 8), (257, 16), (1000, 5), (5000, 12), (300, 20)])
@@ -68,6 +80,16 @@ def test_assign_mean_reconstruct(dtype, width, n, bits):
             want_rg = oracle.reconstruct_backward(go, want_ids, want, groups, relu)
             assert_within(rg, want_rg, **tol)
             assert np.array_equal(rg[small], want_rg[small])
+            if relu:
+                # the same pair with the mask as one bit per element: same rows, the bits of the rows,
+                # and the very sums of the form that reads the rows back
+                for m in (None, members):
+                    rows, signs = abi.reconstruct_signs(_t(grad), ids, None if b is None else _t(b), m)
+                    assert np.array_equal(rows.cpu().numpy(), want)
+                    assert signs.shape == (n, (width + 31) // 32) and signs.dtype == torch.int32
+                    assert np.array_equal(signs.cpu().numpy(), pack_signs(want))
+                rg_bits = abi.reconstruct_backward_signs(_t(go), signs, members, groups).cpu().numpy()
+                assert np.array_equal(rg_bits, rg)
 
 
 @pytest.mark.parametrize("width,bits", [
@@ -212,6 +234,25 @@ def test_large_cluster_sums():
     np.testing.assert_allclose(rg, want, rtol=1e-4, atol=1e-3)
     # the means of the same clusters: unnormalised sums are as large, the quotient is small
     assert_no_less_accurate(reps, oracle.cluster_mean(x, ids_np, counts_np), want64, factor=1.5)
+
+
+def test_sign_bits_of_special_values():
+    """Zero of either sign drops the gradient, NaN and the smallest denormal keep it: the mask
+    `output <= 0` of the reference (cluster_kernel.cu:98-108), bit by bit."""
+    specials = np.array([0.0, -0.0, np.nan, 1e-45, -1e-45, np.inf, -np.inf, 1.0], dtype=np.float32)
+    width = 70
+    reps = np.resize(specials, (3, width)).astype(np.float32)
+    reps[1] = np.roll(reps[0], 3)
+    reps[2] = -reps[0]
+    ids = np.array([2, 0, 1, 1, 0, 2, 2], dtype=np.int64)
+    want = oracle.reconstruct(reps, ids, None, True)
+    rows, signs = abi.reconstruct_signs(_t(reps), _t(ids), None, None)
+    assert np.array_equal(rows.cpu().numpy(), want, equal_nan=True)
+    assert np.array_equal(signs.cpu().numpy(), pack_signs(want))
+    members = abi.cluster_members(_t(ids), 3)
+    go = np.random.default_rng(3).standard_normal((7, width)).astype(np.float32)
+    got = abi.reconstruct_backward_signs(_t(go), signs, members, 3).cpu().numpy()
+    assert np.array_equal(got, oracle.reconstruct_backward(go, ids, want, 3, True))
 
 
 def test_memory_probes_move_what_they_say():

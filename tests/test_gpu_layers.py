@@ -332,6 +332,16 @@ def test_cluster_reconstruct_layers():
                 b = torch.autograd.grad(ref, (reps, bias), go)
                 torch.testing.assert_close(a[0], b[0], atol=1e-5, rtol=1e-4)
                 torch.testing.assert_close(a[1], b[1], atol=1e-5, rtol=1e-4)
+    # what the layer keeps for its backward pass: the index and one bit per element, never the rows
+    reps = torch.randn(5, 100, device=DEV, requires_grad=True)
+    kept = []
+    with torch.autograd.graph.saved_tensors_hooks(lambda t: kept.append(t) or t, lambda t: t):
+        out = reconstruct(reps, idx, activation='relu')
+    assert sorted((tuple(t.shape), t.dtype) for t in kept) == [((6,), torch.int64), ((6, 4), torch.int32)]
+    kept.clear()
+    with torch.autograd.graph.saved_tensors_hooks(lambda t: kept.append(t) or t, lambda t: t):
+        out = reconstruct(reps, idx)
+    assert [tuple(t.shape) for t in kept] == [(6,)]
     reps = torch.randn(5, 3, device=DEV, dtype=torch.double, requires_grad=True)
     bias = torch.full((3,), 2., device=DEV, dtype=torch.double, requires_grad=True)
     assert torch.autograd.gradcheck(lambda a, b: reconstruct(a, idx, b, 'relu'), (reps, bias), eps=1e-6,
@@ -482,6 +492,11 @@ def test_cluster_operators_reject_bad_operands():
         lambda: rt.cluster_reconstruct(reps, ids, torch.zeros(8, device=DEV, dtype=torch.double), False),
         lambda: rt.cluster_reconstruct_backward(torch.zeros(50, 8, device=DEV), ids, torch.zeros(50, 9, device=DEV),
                                                 groups, True),
+        lambda: rt.cluster_reconstruct_signs(reps, ids, torch.zeros(7, device=DEV)),
+        lambda: rt.cluster_reconstruct_backward_signs(torch.zeros(50, 8, device=DEV), ids,
+                                                      torch.zeros(50, 2, device=DEV, dtype=torch.int32), groups),
+        lambda: rt.cluster_reconstruct_backward_signs(torch.zeros(50, 8, device=DEV), ids,
+                                                      torch.zeros(50, 1, device=DEV), groups),  # words are int32
         lambda: rt.cluster_members(ids, 0),
     ]
     for k, call in enumerate(bad_calls):
@@ -496,6 +511,11 @@ def test_cluster_operators_reject_bad_operands():
     for index in (beyond, negative):
         with pytest.raises(RuntimeError, match="outside"):
             rt.cluster_reconstruct(reps, index, None, False)
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_reconstruct_signs(reps, index, None)
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_reconstruct_backward_signs(torch.zeros(50, 8, device=DEV), index,
+                                                  torch.zeros(50, 1, device=DEV, dtype=torch.int32), groups)
         with pytest.raises(RuntimeError, match="outside"):
             rt.cluster_mean_backward(reps, index, counts)
         with pytest.raises(RuntimeError, match="outside"):
