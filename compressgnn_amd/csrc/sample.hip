@@ -76,7 +76,7 @@ __device__ __forceinline__ int64_t draw(uint64_t seed, int64_t layer, int64_t i,
 // The k-th neighbour in the order of storage_api.h:6-70: v2v entries; then, rule by rule of
 // the vertex's v2r entries, the rule's expanded list (its r2v entries, then its children's
 // lists, the children of the wave-th descent taken from level `wave` of r2r).  -1: k lies
-// beyond what the descent finds (the reference throws out_of_range).
+// beyond what the descent finds (the reference throws out_of_range, or reads out of bounds: below).
 __device__ int64_t neighbor_at(const Graph &g, int64_t node, int64_t k) {
     const int64_t v2v_start = g.v2v_ptr[node], v2v_count = g.v2v_ptr[node + 1] - v2v_start;
     if (k < v2v_count) return g.v2v_idx[v2v_start + k];
@@ -102,6 +102,10 @@ __device__ int64_t neighbor_at(const Graph &g, int64_t node, int64_t k) {
             }
             const int64_t own = g.r2v_ptr[rule], own_count = g.r2v_ptr[rule + 1] - own;
             if (k < own_count) return g.r2v_idx[own + k];
+            // The descent found less than r_degree promised (degrees that do not fit the hierarchy).
+            // The reference goes on to the next rule with k - degree, which is negative by now, and
+            // indexes before that rule's list; here the position counts as out of range.
+            return -1;
         }
         k -= degree;
     }

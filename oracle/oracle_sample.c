@@ -59,6 +59,11 @@ static int64_t get_neighbor(const sample_graph *g, int64_t node, int64_t k) {
             }
             const int64_t s = g->r2v_ptr[rule], c = g->r2v_ptr[rule + 1] - s;
             if (k < c) return g->r2v_idx[s + k];
+            /* The descent found fewer entries than r_degree promised (degrees that do not fit the
+             * hierarchy).  storage_api.h:57-64 goes on to the next rule with k - degree < 0 and
+             * indexes before that rule's list (undefined behaviour); when no rule follows it throws
+             * out_of_range.  Here both cases report out of range. */
+            return -1;
         }
         k -= degree;
     }

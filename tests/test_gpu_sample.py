@@ -15,7 +15,7 @@ sys.path[:0] = [os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compr
                 os.path.join(ROOT, "compressgnn_amd", "loader")]
 
 import oracle
-from test_oracle_sample import GOLD, blocks_of, compressed, golden_blocks
+from test_oracle_sample import GOLD, blocks_of, compressed, golden_blocks, misfit_graph
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -75,6 +75,41 @@ def test_sampler_on_deeper_hierarchies():
                 inp = rng.integers(0, V, size=int(rng.integers(1, 12))).astype(np.int64)
                 check(b, dev_blocks, inp, fan, seed=int(rng.integers(0, 10 ** 9)))
         check(b, dev_blocks, np.arange(V, dtype=np.int64), [10 ** 6, 10 ** 6], seed=0)
+
+
+def test_degrees_that_do_not_fit_the_hierarchy():
+    """Expanded degrees larger than what the descent finds: a random position can then fall
+    where the reference would index before a rule's list.  The kernel reports such a position as
+    out of range (IndexError, as the reference's out_of_range) exactly when the oracle does and
+    agrees with it otherwise; nothing is read outside the arrays."""
+    import compressgnn_sample as sampler
+    data = misfit_graph()
+    b = blocks_of(data.edge_index)
+    dev_blocks = on_device(b)
+    V = data.vertex_cnt
+    misfits = np.array([u for u in range(V) if len(oracle.neighbor_list(b, u)) != b["v_degree"][u]], np.int64)
+    assert len(misfits) >= 4
+    rng = np.random.default_rng(17)
+    raised = agreed = 0
+    for case in range(60):
+        inp = np.concatenate([rng.choice(misfits, 6), rng.integers(0, V, 10)]).astype(np.int64)
+        fan = [int(rng.choice([1, 2, 5])) for _ in range(int(rng.integers(1, 3)))]
+        seed = int(rng.integers(0, 2 ** 40))
+        try:
+            want = oracle.neighbor_sample(b, inp, fan, seed=seed)
+        except IndexError:
+            want = None
+        if want is None:
+            with pytest.raises(IndexError, match="out of range"):
+                sampler.neighbor_sample_cg_sim(*dev_blocks, torch.from_numpy(inp).to(DEV), fan, seed=seed)
+            raised += 1
+        else:
+            got = sampler.neighbor_sample_cg_sim(*dev_blocks, torch.from_numpy(inp).to(DEV), fan, seed=seed)
+            assert all(np.array_equal(a.cpu().numpy(), w) for a, w in zip(got, want)), (fan, seed)
+            agreed += 1
+    assert raised >= 3 and agreed >= 3, (raised, agreed)
+    # full lists (fan-out beyond every degree) never descend by position: same lists as the oracle
+    check(b, dev_blocks, np.arange(V, dtype=np.int64), [10 ** 6], seed=2)
 
 
 def test_plain_form_and_large_fanouts():

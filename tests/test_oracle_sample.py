@@ -65,6 +65,42 @@ def compressed(kind, seed=3):
     return data, np.asarray(v, np.int64), np.asarray(e, np.int64)
 
 
+def misfit_graph():
+    """A graph of two rule levels on which some expanded degrees exceed what the descent of
+    get_neighbor finds (the reference's degrees do not cover every hierarchy): 500-vertex copy
+    model, pairs merged from frequency 3 on, no threshold filter, depth limit 8."""
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    v, e = off.gen_copy_model(500, 9.8, 0.7, 1)
+    m = np.ones(500, bool)
+    data = CompressgnnData(np.zeros((500, 1), np.float32), (v, e), np.zeros(500, np.int64), m, m, m, add_self_loop=True,
+                           normalize=False, graph_type="csr", min_pair_frequency=3, threshold=0, max_depth=8, min_edge=0,
+                           verbose=False)
+    return data
+
+
+def test_positions_the_descent_cannot_resolve_are_out_of_range():
+    """Where r_degree promises more than a rule's descent finds, storage_api.h:57-64 goes on to the next
+    rule with a negative position and indexes before that rule's list (or throws when no rule
+    follows).  The oracle reports every such position as out of range and never leaves the arrays."""
+    data = misfit_graph()
+    b = blocks_of(data.edge_index)
+    assert data.edge_index.step >= 2
+    lost = []
+    for u in range(data.vertex_cnt):
+        k = np.arange(b["v_degree"][u])
+        got = oracle.get_neighbors(b, np.full(len(k), u), k)
+        assert ((got >= 0) | (got == -1)).all() and (got < data.vertex_cnt).all()
+        lost += [(u, int(p)) for p in k[got < 0]]
+    assert len(lost) >= 5
+    # the sampler raises when the selection loop draws such a position
+    u, p = lost[0]
+    with pytest.raises(IndexError):
+        oracle.neighbor_sample(b, np.array([u], np.int64), [1], draw=lambda high: min(p, high - 1))
+    # and samples as usual around it
+    oracle.neighbor_sample(b, np.array([u], np.int64), [1], draw=lambda high: 0)
+
+
 def test_golden_vectors_of_the_compiled_reference():
     g = np.load(os.path.join(GOLD, "sample_golden.npz"))
     off = np.load(os.path.join(GOLD, "offline_golden.npz"))
