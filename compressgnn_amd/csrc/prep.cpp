@@ -970,20 +970,27 @@ cgnn_arrays *cgnn_csr_locality_order(int64_t rows, const int64_t *vlist, const i
 #else
         std::sort(lex.begin(), lex.end(), before);
 #endif
-        // column -> rows that list it
-        i64 cols = 0;
+        // column -> rows that list it.  Scattered counting and filling are most of the time of
+        // this function on graphs beyond the caches, so all cores take part; the rows of a
+        // column then stand in no particular order, which the matching below does not read.
+        i64 cols = 0, lowest = 0;
+#pragma omp parallel for reduction(max : cols) reduction(min : lowest) schedule(static)
         for (i64 e = 0; e < nnz; ++e) {
-            if (elist[e] < 0) throw std::runtime_error("csr_locality_order: negative column");
             cols = std::max(cols, elist[e] + 1);
+            lowest = std::min(lowest, elist[e]);
         }
+        if (lowest < 0) throw std::runtime_error("csr_locality_order: negative column");
         std::vector<i64> cstart((size_t)cols + 1, 0);
-        for (i64 e = 0; e < nnz; ++e) ++cstart[elist[e] + 1];
+#pragma omp parallel for schedule(static)
+        for (i64 e = 0; e < nnz; ++e) __atomic_fetch_add(&cstart[elist[e] + 1], (i64)1, __ATOMIC_RELAXED);
         for (i64 c = 0; c < cols; ++c) cstart[c + 1] += cstart[c];
         std::vector<int32_t> crow((size_t)nnz);
         {
             std::vector<i64> fill(cstart.begin(), cstart.end() - 1);
+#pragma omp parallel for schedule(static)
             for (i64 r = 0; r < rows; ++r)
-                for (i64 e = vlist[r]; e < vlist[r + 1]; ++e) crow[fill[elist[e]]++] = (int32_t)r;
+                for (i64 e = vlist[r]; e < vlist[r + 1]; ++e)
+                    crow[__atomic_fetch_add(&fill[elist[e]], (i64)1, __ATOMIC_RELAXED)] = (int32_t)r;
         }
         i64 hub_rows = kLocalityHubRows;
         for (; hub_rows > 2; hub_rows /= 2) {
