@@ -208,8 +208,8 @@ int cgnn_lsh_scan(int bits, const int32_t *bucket_count, int32_t *prefix, void *
 int cgnn_lsh_finish(int64_t N, int bits, const int32_t *raw_code, const int32_t *bucket_count,
                     const int32_t *prefix, int64_t *ids, int32_t *counts, cgnn_stream_t stream);
 
-/* The bad_id argument of the three entries that read caller-supplied cluster ids
- * (cgnn_cluster_members, cgnn_cluster_mean_backward, cgnn_reconstruct): a device int32, or
+/* The bad_id argument of the entries that read caller-supplied cluster ids
+ * (cgnn_cluster_members, cgnn_cluster_mean_backward, cgnn_reconstruct, cgnn_reconstruct_signs): a device int32, or
  * NULL.  The reference traps in the kernel on an id outside [0, groups)
  * (CUDA_KERNEL_ASSERT, cluster_kernel.cu:74,92); here such an id is treated as the nearest
  * valid one, so that no access leaves the arrays, and 1 is stored to *bad_id.  0 is never
