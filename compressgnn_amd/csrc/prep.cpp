@@ -307,16 +307,20 @@ cgnn_arrays *emit_filtered(const EditedRows &g, const std::vector<char> &dropped
         new_id[r] = next;
         if (!dropped[r]) ++next;
     }
-    i64 total = 0;
-    for (i64 n = 0; n < V + R; ++n)
-        if (n < V || !dropped[n - V]) total += g.size_of(n);
-    std::vector<i64> nv{0}, ne;
-    nv.reserve(next + 1);
-    ne.reserve(total);
+    // where every surviving row starts, then all cores copy rows (most of a filter pass on a
+    // large graph is this copy)
+    std::vector<i64> nv((size_t)next + 1, 0);
     for (i64 n = 0; n < V + R; ++n) {
         if (n >= V && dropped[n - V]) continue;
-        g.for_each(n, [&](i64 c) { ne.push_back(c >= V ? new_id[c - V] : c); });
-        nv.push_back((i64)ne.size());
+        const i64 k = n < V ? n : new_id[n - V];
+        nv[k + 1] = nv[k] + g.size_of(n);
+    }
+    std::vector<i64> ne((size_t)nv[next]);
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < V + R; ++n) {
+        if (n >= V && dropped[n - V]) continue;
+        i64 at = nv[n < V ? n : new_id[n - V]];
+        g.for_each(n, [&](i64 c) { ne[at++] = c >= V ? new_id[c - V] : c; });
     }
     auto *out = new cgnn_arrays;
     out->add(std::move(nv));

@@ -102,8 +102,24 @@ class CompressgnnData():
         # gen_mask_vertex(..., "csc"), :177-179); the kernels go by CompressGraph.step
         self.step = offline.gen_vertex_order_csc(vlist, elist, self.vertex_cnt, self.rule_cnt)[1]
         nodes = self.vertex_cnt + self.rule_cnt
-        colptr, row, value = offline.csr_transpose(vlist, elist, weight, nodes)
+        colptr, row, value = self._by_column(vlist, elist, weight, nodes)
         self.edge_index = CompressGraph(colptr, row, value, self.vertex_cnt)
+
+    def _by_column(self, vlist, elist, weight, nodes):
+        """The compressed matrix by column (SparseTensor.csc() of the reference, :180): on the GPU
+        when the loader already works there (compression_backend 'cuda'), the same arrays bit for
+        bit as the host routine; a graph that does not fit the device beside what is there goes to
+        the host routine."""
+        if self.compression_backend == 'cuda':
+            import compressgnn_runtime as rt
+            dev = torch.device('cuda', torch.cuda.current_device())
+            try:
+                parts = rt.csr_transpose(torch.from_numpy(vlist).to(dev), torch.from_numpy(elist).to(dev),
+                                         torch.from_numpy(weight).to(dev), nodes)
+                return tuple(p.cpu().numpy() for p in parts)
+            except torch.cuda.OutOfMemoryError:
+                pass
+        return offline.csr_transpose(vlist, elist, weight, nodes)
 
     # graph_type="coo": (src, dst) -> edge and weight tensors per phase  (:86-139)
     def _from_edges(self, src, dst, add_self_loop, normalize, verbose):

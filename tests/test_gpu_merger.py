@@ -98,3 +98,24 @@ def test_gpu_compressor_rejects_bad_input_and_is_the_loaders_choice():
     a = compression_backend.compress_graph_csr(v, e, 16, backend="cuda")
     b = compression_backend.compress_graph_csr(v, e, 16, backend="cpu")
     assert all(np.array_equal(x, y) for x, y in zip(a[:2], b[:2])) and a[2:] == b[2:]
+
+
+def test_loader_gives_the_same_dataset_on_either_backend():
+    """CompressgnnData with the work on the GPU (rule merger and the by-column form of the
+    compressed matrix) holds the same blocks, weights and degrees as with everything on the host."""
+    sys.path.insert(0, os.path.join(ROOT, "compressgnn_amd", "layer"))
+    from compressgnn_amd import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    v, e = off.gen_copy_model(20000, 9.8, 0.7, 11)
+    V = len(v) - 1
+    m = np.ones(V, bool)
+    both = [CompressgnnData(np.zeros((V, 1), np.float32), (v, e), np.zeros(V, np.int64), m, m, m, graph_type="csr",
+                            min_pair_frequency=4, compression_backend=backend, verbose=False) for backend in ("cuda", "cpu")]
+    a, b = (d.edge_index for d in both)
+    assert (both[0].vertex_cnt, both[0].rule_cnt, both[0].edge_cnt, a.step) == (both[1].vertex_cnt, both[1].rule_cnt, both[1].edge_cnt, b.step)
+    assert both[0].rule_cnt > 0
+    for x, y in zip(a.blocks(), b.blocks()):
+        for p, q in zip(x.csr(), y.csr()):
+            assert p.dtype == q.dtype and np.array_equal(p.cpu().numpy(), q.cpu().numpy())
+    assert np.array_equal(a.vertex_degree.numpy(), b.vertex_degree.numpy())
+    assert np.array_equal(a.rule_degree.numpy(), b.rule_degree.numpy())
