@@ -12,6 +12,7 @@
 
 #include <memory>
 #include <sstream>
+#include <map>
 #include <string>
 #include <tuple>
 #include <vector>
@@ -255,6 +256,10 @@ struct StageTimer {
     };
     std::vector<std::string> timed;
     std::vector<Rec> recs;
+    // An event pair costs the stream a few microseconds of idle time on either side of the stage, so
+    // a caller that times a loop may ask for every n-th pass of a stage only.
+    int64_t every = 1;
+    std::map<std::string, int64_t> passes;
 
     bool wants(const std::string &name) const {
         for (auto &t : timed)
@@ -263,6 +268,7 @@ struct StageTimer {
     }
     int open(const std::string &name, hipStream_t stream) {
         if (!wants(name)) return -1;
+        if (passes[name]++ % std::max<int64_t>(every, 1) != 0) return -1;
         Rec r{name, nullptr, nullptr};
         TORCH_CHECK(hipEventCreate(&r.begin) == hipSuccess && hipEventCreate(&r.end) == hipSuccess, "hipEventCreate failed");
         TORCH_CHECK(hipEventRecord(r.begin, stream) == hipSuccess, "hipEventRecord failed");
@@ -1033,6 +1039,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
                       [](PropagationPlan &p, std::string mth) { p.kernel = kernel_of_method(mth); })
         .def_property("timed_stages", [](PropagationPlan &p) { return p.timer.timed; },
                       [](PropagationPlan &p, std::vector<std::string> names) { p.timer.timed = names; })
+        .def_property("timed_every", [](PropagationPlan &p) { return p.timer.every; },
+                      [](PropagationPlan &p, int64_t n) {
+                          TORCH_CHECK(n >= 1, "timed_every must be at least 1");
+                          p.timer.every = n;
+                          p.timer.passes.clear();
+                      })
         .def("take_stage_times", [](PropagationPlan &p) { return p.timer.take(); })
         .def_readonly("v2v", &PropagationPlan::v2v)
         .def_readonly("v2r", &PropagationPlan::v2r)
