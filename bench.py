@@ -19,6 +19,7 @@ resident in HBM.  Prints ONE JSON line:
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cluster] [--skip-cpu] [--skip-sweep] [--skip-c4]
        python bench.py --c4 [--c4-vertices N]   (the large end-to-end configuration only)
+       python bench.py --probe read|write|copy [--probe-mib M] [--probe-launches K]   (memory ceilings only)
 """
 import argparse
 import json
@@ -423,6 +424,30 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
     }
 
 
+def memory_probe(torch, mode, mib, launches):
+    """The library's plain copy (cgnn_copy_bytes), streaming-read (cgnn_read_bytes) or
+    streaming-write (cgnn_fill_bytes) kernel over a buffer of known size, timed with HIP events.
+    A buffer that fits the 256 MB last-level cache shows what that cache delivers, a larger one
+    what HBM delivers."""
+    import ctypes
+    from compressgnn_amd import abi
+    n = mib << 20
+    src = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+    L = abi.lib()
+    if mode == "read":
+        sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+        run = lambda: abi.check(L.cgnn_read_bytes(abi.ptr(src), ctypes.c_size_t(n), abi.ptr(sink), abi.stream_of(src)))
+    elif mode == "write":
+        run = lambda: abi.check(L.cgnn_fill_bytes(abi.ptr(src), ctypes.c_size_t(n), abi.stream_of(src)))
+    else:
+        dst = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+        run = lambda: abi.check(L.cgnn_copy_bytes(abi.ptr(src), abi.ptr(dst), ctypes.c_size_t(n), abi.stream_of(src)))
+    ms = time_loop(run, launches, 1, torch)
+    moved = n if mode in ("read", "write") else 2 * n
+    print("%s: %d bytes per launch x %d launches, %.1f us per launch, %.0f GB/s (%s)"
+          % (mode, n, launches, ms * 1e3, moved / ms / 1e6, mode if mode in ("read", "write") else "read + write"))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -434,10 +459,12 @@ def main():
     ap.add_argument("--skip-sweep", action="store_true", help="leave out the feature sweep F in {16, 64, 256, 512} (C2)")
     ap.add_argument("--skip-c4", action="store_true",
                     help="leave out the large end-to-end leg (C4: about two minutes of graph preparation)")
-    ap.add_argument("--windowed-probe", action="store_true",
-                    help="also time the kernels on a graph with the row lengths of C1 whose gathers stay in L2")
-    ap.add_argument("--stream-rows-over", type=int, default=0,
-                    help="forward vertex stage: streaming loads for the runs of rows longer than this (0 = off)")
+    ap.add_argument("--probe", choices=["read", "write", "copy"],
+                    help="run only the library's plain streaming kernel over a buffer of --probe-mib MiB, "
+                         "--probe-launches times, and print its rate (the ceilings the kernels are compared with; under "
+                         "rocprofv3 --pmc the copy gives the factor that turns FETCH_SIZE / WRITE_SIZE into bytes)")
+    ap.add_argument("--probe-mib", type=int, default=1024)
+    ap.add_argument("--probe-launches", type=int, default=3)
     ap.add_argument("--c4", action="store_true",
                     help="run only the large end-to-end configuration (2-layer GCN epoch) and print its line")
     ap.add_argument("--c4-vertices", type=int, default=C4_VERTICES)
@@ -452,6 +479,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     import compressgnn_runtime as rt
     from CompressgnnSPMM import compress_spmm  # noqa: F401  (the layer path uses the same plan)
+    if args.probe:
+        memory_probe(torch, args.probe, args.probe_mib, args.probe_launches)
+        return
     if args.c4:
         print(json.dumps(bench_c4(torch, args.c4_vertices, args.c4_epochs, args.c4_refresh_interval)))
         return
@@ -463,7 +493,6 @@ def main():
     acct = graph_accounting(graph, F)
     data.to(dev)
     plan = graph.plan()
-    plan.vertex_stage.stream_rows_over = args.stream_rows_over
     gen = torch.Generator(device=dev)
     gen.manual_seed(7)
     x = torch.randn(C1_VERTICES, F, device=dev, generator=gen)
@@ -497,22 +526,21 @@ def main():
                                              forward_GBps=pb_f["bytes"] / (f_ms * 1e-3) / 1e9,
                                              backward_GBps=pb_b["bytes"] / (b_ms * 1e-3) / 1e9,
                                              forward_bytes=pb_f["bytes"], backward_bytes=pb_b["bytes"])
-    if args.windowed_probe:
-        # the same kernels on a graph whose gathers stay in L2: row lengths and weights of the C1 graph,
-        # neighbours drawn from a window of 2,048 vertices around the row instead of the copy model
-        rng_l = np.random.default_rng(11)
-        src_l = np.repeat(np.arange(C1_VERTICES, dtype=np.int64), np.diff(v2))
-        col_l = (src_l + rng_l.integers(-1024, 1024, size=len(src_l))) % C1_VERTICES
-        col_l = col_l[np.argsort(src_l * C1_VERTICES + col_l, kind="stable")]
-        local = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(col_l), torch.from_numpy(w), C1_VERTICES,
-                             C1_VERTICES, dev)
-        lb = block_bytes(v2, col_l, C1_VERTICES, F, 0)
-        early["windowed_graph_same_row_lengths"] = {}
-        for name, forced in (("rowbalance", "row_schedule"), ("nnzbalance", "nnz_schedule")):
-            l_ms = time_loop(lambda: local.spmm(x, None, forced), args.steps, 2, torch)
-            early["windowed_graph_same_row_lengths"][name] = dict(ms=l_ms, bytes=lb["bytes"],
-                                                                   GBps=lb["bytes"] / (l_ms * 1e-3) / 1e9)
-        del local
+    # the same kernels on a graph whose gathers stay in L2: row lengths and weights of the C1 graph,
+    # neighbours drawn from a window of 2,048 vertices around the row instead of the copy model
+    rng_l = np.random.default_rng(11)
+    src_l = np.repeat(np.arange(C1_VERTICES, dtype=np.int64), np.diff(v2))
+    col_l = (src_l + rng_l.integers(-1024, 1024, size=len(src_l))) % C1_VERTICES
+    col_l = col_l[np.argsort(src_l * C1_VERTICES + col_l, kind="stable")]
+    local = rt.DeviceCsr(torch.from_numpy(v2), torch.from_numpy(col_l), torch.from_numpy(w), C1_VERTICES,
+                         C1_VERTICES, dev)
+    lb = block_bytes(v2, col_l, C1_VERTICES, F, 0)
+    early["windowed_graph_same_row_lengths"] = {}
+    for name, forced in (("rowbalance", "row_schedule"), ("nnzbalance", "nnz_schedule")):
+        l_ms = time_loop(lambda: local.spmm(x, None, forced), args.steps, 2, torch)
+        early["windowed_graph_same_row_lengths"][name] = dict(ms=l_ms, bytes=lb["bytes"],
+                                                               GBps=lb["bytes"] / (l_ms * 1e-3) / 1e9)
+    del local
     # parity of the measured configuration: compressed == plain within tolerance
     out, gx = step()
     ref_out = plain_t.spmm(x, None, "row_schedule")

@@ -18,7 +18,7 @@ SPMM_AUTO, SPMM_ROW, SPMM_NNZ = 0, 1, 2
 EXPORTS = [
     "cgnn_last_error", "cgnn_version",
     "cgnn_spmm_schedule", "cgnn_spmm_run_length", "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
-    "cgnn_spmm_static_scratch_bytes", "cgnn_spmm_static",
+    "cgnn_spmm_static_scratch_bytes", "cgnn_spmm_static_init", "cgnn_spmm_static",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
     "cgnn_csr_transpose_workspace_bytes", "cgnn_csr_transpose_device",
     "cgnn_compress_batch_workspace_bytes", "cgnn_compress_csr_batch_device",
@@ -38,7 +38,7 @@ class CsrStruct(ctypes.Structure):
         ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("nnz", ctypes.c_int64),
         ("rowptr", ctypes.c_void_p), ("colidx", ctypes.c_void_p), ("rowidx", ctypes.c_void_p),
         ("val", ctypes.c_void_p), ("max_row_nnz", ctypes.c_int32), ("seg_nnz", ctypes.c_int32),
-        ("rowmap", ctypes.c_void_p), ("stream_rows_over", ctypes.c_int32),
+        ("rowmap", ctypes.c_void_p),
         ("cut_rows", ctypes.c_void_p), ("empty_rows", ctypes.c_void_p),
         ("n_cut_rows", ctypes.c_int32), ("n_empty_rows", ctypes.c_int32),
     ]

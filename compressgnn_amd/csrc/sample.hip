@@ -189,8 +189,10 @@ __global__ __launch_bounds__(kBlock) void sample_count_kernel(LayerArgs a) {
                 const int64_t full = full_list_sizes(a.g, node, per_depth);
                 if (full >= INT32_MAX) *a.status = CGNN_SAMPLE_TOO_MANY;
                 else count = (int32_t)full;
+            } else if (a.fanout >= INT32_MAX) {
+                *a.status = CGNN_SAMPLE_TOO_MANY;  // one vertex alone would add 2^31 - 1 neighbours or more
             } else {
-                count = (int32_t)a.fanout;  // fanout < degree < 2^31 is checked on the host
+                count = (int32_t)a.fanout;
             }
         }
     }

@@ -90,7 +90,6 @@ struct SpmmArgs {
     int32_t stretch_log2;  // log2 of the workgroups per XCD stretch (see logical_block); set at launch
     int32_t blocks;        // workgroups with work (the grid rounds this up to a multiple of kXcds)
     int32_t read_once;     // MODE_UNIT: every row of X is gathered once (member lists), so with streaming loads
-    int32_t stream_over;   // nnz schedule: runs inside a row of more entries than this gather with streaming loads (0: none)
     const int32_t *cut_rows;    // spmm_fixup_rows_kernel: the stored rows that the runs cut, ascending
     const int32_t *empty_rows;  // and the stored rows without entries
     int32_t n_cut_rows, n_empty_rows;
@@ -229,7 +228,7 @@ __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_
 // Gather one feature tile of column c (source chosen by `src` in MODE_DUAL, masked by
 // M in MODE_RELU_MASK and by the bits of `signs` in MODE_SIGN_MASK).
 template <typename T, int VEC, int MODE>
-__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int src, int64_t foff, bool stream = false) {
+__device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int src, int64_t foff) {
     Pack<T, VEC> x;
     if (foff < 0) {
 #pragma unroll
@@ -245,8 +244,7 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
     }
     const int64_t off = (int64_t)c * (int32_t)a.F + foff;  // F < 2^31: one 32 x 32 -> 64 bit multiply
     // rows that are gathered once (member lists; masks exist for those only) are not kept in the caches
-    // (`stream`: the same for the runs of hub rows of a graph block when the block asks for it; uniform over the wave)
-    if (MODE == MODE_RELU_MASK || MODE == MODE_SIGN_MASK || (MODE == MODE_UNIT && a.read_once) || stream)
+    if (MODE == MODE_RELU_MASK || MODE == MODE_SIGN_MASK || (MODE == MODE_UNIT && a.read_once))
         x = load_pack_stream<T, VEC>(base + off);
     else
         x = load_pack<T, VEC>(base + off);
@@ -443,17 +441,6 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     acc.clear();
     int cur = -1;
     bool continues = false;
-    // Hub rows: when every run of this wave lies inside a row of more than stream_over entries,
-    // its gathers do not displace lines that the short rows around them come back to.
-    bool stream = false;
-    if (a.stream_over > 0) {
-        bool hub = true;
-        if (active) {
-            const int first = a.rowidx[e0];
-            hub = first == a.rowidx[e1 - 1] && a.rowptr[first + 1] - a.rowptr[first] > a.stream_over;
-        }
-        stream = __ballot(!hub) == 0;
-    }
     if (active) {
         cur = a.rowidx[e0];
         if constexpr (LPR >= kUnroll && sizeof(T) == 4) {
@@ -498,7 +485,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                             if (u0 + u < cnt) {
 #pragma unroll
                                 for (int t = 0; t < TILES; ++t)
-                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t], stream);
+                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
                             }
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u) {
@@ -1102,7 +1089,6 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
         a.M = nullptr;
         M = nullptr;
     }
-    a.stream_over = A->stream_rows_over > 0 ? A->stream_rows_over : 0;
     kernel = resolve_kernel(A, kernel);
     if (masked) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
     if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;
@@ -1262,6 +1248,11 @@ extern "C" int cgnn_spmm_schedule(int64_t rows, int64_t nnz, int32_t max_row_nnz
 extern "C" int cgnn_spmm_run_length(const cgnn_csr *A) { return A == nullptr ? 0 : seg_len(A); }
 
 extern "C" size_t cgnn_spmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int cgnn_spmm_static_init(void) {
+    void *ws = nullptr;
+    return static_scratch(&ws);
+}
 
 extern "C" int cgnn_spmm_static(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F, int accumulate,
                                 int kernel, cgnn_stream_t stream) {

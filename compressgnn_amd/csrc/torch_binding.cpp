@@ -10,7 +10,9 @@
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
+#include <deque>
 #include <memory>
+#include <mutex>
 #include <sstream>
 #include <map>
 #include <string>
@@ -65,7 +67,6 @@ struct DeviceCsr {
     Tensor rowmap;  // optional: stored row g is output row rowmap[g]
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
-    int32_t stream_rows_over = 0;
     Tensor cut_rows, empty_rows;  // the rows the runs of the nnz schedule cut / the rows without entries
     std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
 
@@ -81,7 +82,6 @@ struct DeviceCsr {
         a.max_row_nnz = max_row_nnz;
         a.seg_nnz = seg_nnz;
         a.rowmap = rowmap.defined() ? rowmap.data_ptr<int32_t>() : nullptr;
-        a.stream_rows_over = stream_rows_over;
         if (cut_rows.defined()) {
             a.cut_rows = cut_rows.data_ptr<int32_t>();  // a tensor without entries gives a pointer that is never read
             a.n_cut_rows = (int32_t)cut_rows.numel();
@@ -502,6 +502,54 @@ std::tuple<Tensor, Tensor, int64_t, std::vector<Tensor>> cluster_assign_members(
             {offsets.narrow(0, 0, active + 2), perm, sorted_id, host_scalar(summary.data_ptr<int32_t>()[1])}};
 }
 
+// Member lists by the index tensor they belong to.  The operators with the reference's
+// signatures (cluster_mean(input, index, count), cluster_reconstruct(reps, index, bias, relu), ...)
+// receive an index and nothing else; the lists that go with it, and the knowledge that its ids
+// were checked, are kept here so that only the first call on an index builds them (one host
+// read), as the reference reads the host once per assignment (cluster_kernel.cu:147).  An entry
+// names its tensor by a weak reference and the tensor's version counter: it is dropped when the
+// tensor is freed and ignored once the tensor was written to.
+struct MemberCache {
+    struct Entry {
+        c10::weak_intrusive_ptr<c10::TensorImpl> index;
+        uint32_t version;
+        int64_t groups;
+        std::vector<Tensor> members;
+    };
+    static constexpr size_t kKeep = 8;
+    std::deque<Entry> entries;
+    std::mutex lock;
+
+    bool find(const Tensor &index, int64_t groups, std::vector<Tensor> *out) {
+        std::lock_guard<std::mutex> hold(lock);
+        for (auto it = entries.begin(); it != entries.end();) {
+            if (it->index.expired()) {
+                it = entries.erase(it);
+                continue;
+            }
+            if (it->index._unsafe_get_target() == index.unsafeGetTensorImpl() && it->version == index._version() &&
+                (groups < 0 || it->groups == groups)) {
+                *out = it->members;
+                return true;
+            }
+            ++it;
+        }
+        return false;
+    }
+    void put(const Tensor &index, int64_t groups, std::vector<Tensor> members) {
+        if (index.is_inference()) return;  // no version counter to tell a later write by
+        std::lock_guard<std::mutex> hold(lock);
+        entries.push_front(Entry{c10::weak_intrusive_ptr<c10::TensorImpl>(index.getIntrusivePtr()), index._version(),
+                                 groups, std::move(members)});
+        while (entries.size() > kKeep) entries.pop_back();
+    }
+};
+
+MemberCache &member_cache() {
+    static MemberCache cache;
+    return cache;
+}
+
 // cluster_assign_cuda (cluster_kernel.cu:118-153).  The three tensors of cluster_workspace
 // are accepted, and must be what cluster_workspace returns for these arguments; the grouping
 // itself sorts the codes and no longer touches bucket counters.
@@ -522,6 +570,9 @@ std::tuple<Tensor, Tensor, int64_t> cluster_assign(Tensor input, Tensor planes, 
                     w.defined() ? seen(w) : "undefined");
     }
     auto grouped = cluster_assign_members(input, planes, bits);
+    // the lists made along the way stay with the ids: the operators that are handed these ids
+    // (and nothing else) find them again
+    member_cache().put(std::get<0>(grouped), std::get<2>(grouped) + 1, std::get<3>(grouped));
     return {std::get<0>(grouped), std::get<1>(grouped), std::get<2>(grouped)};
 }
 
@@ -587,9 +638,15 @@ void expect_members(const char *op, const std::vector<Tensor> &m, const Tensor &
 
 std::vector<Tensor> members_or_build(const char *op, const c10::optional<std::vector<Tensor>> &members,
                                      const Tensor &index, int64_t groups) {
-    if (!has_members(members)) return cluster_members(index, groups);
-    expect_members(op, *members, index, groups);
-    return *members;
+    if (has_members(members)) {
+        expect_members(op, *members, index, groups);
+        return *members;
+    }
+    std::vector<Tensor> known;
+    if (member_cache().find(index, groups, &known)) return known;
+    known = cluster_members(index, groups);  // checks the ids: the one host read for this index
+    member_cache().put(index, groups, known);
+    return known;
 }
 
 int64_t largest_group(const std::vector<Tensor> &m) { return m.size() == 4 ? m[3].item<int64_t>() : 0; }
@@ -614,13 +671,26 @@ Tensor cluster_mean(Tensor input, Tensor index, Tensor count, c10::optional<std:
     return out;
 }
 
-// The order in which a gather produces its rows: the member list `perm` when the caller has one.
-// An index that comes without member lists is an index from outside the assignment operators,
-// and its ids are checked (one host read).
-const int32_t *production_order(const char *op, const c10::optional<std::vector<Tensor>> &members, const Tensor &index) {
-    if (!has_members(members)) return nullptr;
-    expect_members(op, *members, index, -1);
-    return (*members)[1].data_ptr<int32_t>();
+// The order in which a gather produces its rows: the member list `perm` when the caller has one
+// or an earlier operator on the same index has left one (`held` keeps it alive for the call).
+// An index met for the first time, without lists, is an index from outside the assignment
+// operators: its ids are checked by the gather itself (one host read) and its lists are built
+// for the calls that follow.
+const int32_t *production_order(const char *op, const c10::optional<std::vector<Tensor>> &members, const Tensor &index,
+                                int64_t groups, std::vector<Tensor> *held) {
+    if (has_members(members)) {
+        expect_members(op, *members, index, -1);
+        return (*members)[1].data_ptr<int32_t>();
+    }
+    if (member_cache().find(index, groups, held)) return (*held)[1].data_ptr<int32_t>();
+    return nullptr;
+}
+
+// After a gather over an index that had no lists: the flag is read (the ids are then known to be
+// good) and the lists are made, so that later operators on this index read nothing.
+void remember_checked_index(const char *op, IdFlag &bad, const Tensor &index, int64_t groups) {
+    bad.raise(op, groups);
+    if (groups >= 1) member_cache().put(index, groups, cluster_members(index, groups));
 }
 
 // cluster_mean_backward_cuda (cluster_kernel.cu:171-181).
@@ -631,14 +701,15 @@ Tensor cluster_mean_backward(Tensor grad, Tensor index, Tensor count, c10::optio
     c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
     Tensor out = torch::empty({index.numel(), grad.size(1)}, grad.options());
     if (out.numel() == 0) return out;
-    const int32_t *perm = production_order(op, members, index);
+    std::vector<Tensor> held;
+    const int32_t *perm = production_order(op, members, index, count.numel(), &held);
     c10::optional<IdFlag> bad;
     if (perm == nullptr) bad.emplace(index);
     ok(cgnn_cluster_mean_backward(index.numel(), grad.size(1), count.numel(), dtype_code(grad), grad.data_ptr(),
                                   index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), perm, out.data_ptr(),
                                   bad ? bad->ptr() : nullptr, current_stream(grad)),
        op);
-    if (bad) bad->raise(op, count.numel());
+    if (bad) remember_checked_index(op, *bad, index, count.numel());
     return out;
 }
 
@@ -655,14 +726,15 @@ Tensor cluster_reconstruct(Tensor reps, Tensor index, c10::optional<Tensor> bias
     c10::hip::HIPGuardMasqueradingAsCUDA guard(reps.device());
     Tensor out = torch::empty({index.numel(), reps.size(1)}, reps.options());
     if (out.numel() == 0) return out;
-    const int32_t *perm = production_order(op, members, index);
+    std::vector<Tensor> held;
+    const int32_t *perm = production_order(op, members, index, reps.size(0), &held);
     c10::optional<IdFlag> bad;
     if (perm == nullptr) bad.emplace(index);
     ok(cgnn_reconstruct(index.numel(), reps.size(1), reps.size(0), dtype_code(reps), reps.data_ptr(),
                         index.data_ptr<int64_t>(), perm, bias.has_value() ? bias->data_ptr() : nullptr, relu ? 1 : 0,
                         out.data_ptr(), bad ? bad->ptr() : nullptr, current_stream(reps)),
        op);
-    if (bad) bad->raise(op, reps.size(0));
+    if (bad) remember_checked_index(op, *bad, index, reps.size(0));
     return out;
 }
 
@@ -705,7 +777,8 @@ std::tuple<Tensor, Tensor> cluster_reconstruct_signs(Tensor reps, Tensor index, 
     Tensor out = torch::empty({N, F}, reps.options());
     Tensor signs = torch::empty({N, cgnn_sign_words(F)}, reps.options().dtype(torch::kInt32));
     if (out.numel() == 0) return {out, signs};
-    const int32_t *perm = production_order(op, members, index);
+    std::vector<Tensor> held;
+    const int32_t *perm = production_order(op, members, index, reps.size(0), &held);
     c10::optional<IdFlag> bad;
     if (perm == nullptr) bad.emplace(index);
     ok(cgnn_reconstruct_signs(N, F, reps.size(0), dtype_code(reps), reps.data_ptr(), index.data_ptr<int64_t>(), perm,
@@ -713,7 +786,7 @@ std::tuple<Tensor, Tensor> cluster_reconstruct_signs(Tensor reps, Tensor index, 
                               reinterpret_cast<uint32_t *>(signs.data_ptr<int32_t>()), bad ? bad->ptr() : nullptr,
                               current_stream(reps)),
        op);
-    if (bad) bad->raise(op, reps.size(0));
+    if (bad) remember_checked_index(op, *bad, index, reps.size(0));
     return {out, signs};
 }
 
@@ -983,7 +1056,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
                       })
         .def_readonly("cut_rows", &DeviceCsr::cut_rows)
         .def_readonly("empty_rows", &DeviceCsr::empty_rows)
-        .def_readwrite("stream_rows_over", &DeviceCsr::stream_rows_over)
         .def_readonly("rowptr", &DeviceCsr::rowptr)
         .def_readonly("colidx", &DeviceCsr::colidx)
         .def_readonly("rowidx", &DeviceCsr::rowidx)

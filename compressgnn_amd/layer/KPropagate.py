@@ -9,7 +9,6 @@ import _paths  # noqa: F401
 from torch import Tensor
 
 from CompressgnnPropagation import Propagate
-from type import OptTensor
 
 
 class HopLayer(Propagate):
@@ -21,12 +20,6 @@ class HopLayer(Propagate):
         for _ in range(count):
             x = self.compressgnn_propagate(x, edge_index, edge_weight, None, vertex_cnt, rule_cnt)
         return x
-
-    def message(self, x_j: Tensor, edge_weight: OptTensor) -> Tensor:
-        # the source row, scaled by the weight of the edge when there is one
-        if edge_weight is None:
-            return x_j
-        return x_j * edge_weight.view(-1, 1)
 
 
 class KPropagate(HopLayer):

@@ -66,11 +66,6 @@ typedef struct cgnn_csr {
      * of such a block are numbered so that consecutive stored rows land on the same XCD
      * (the eight L2 caches of an MI355X are private). */
     const int32_t *rowmap; /* [rows] or NULL */
-    /* NNZ schedule, optional (0 = off): runs that lie inside a row of more than this many
-     * entries gather their rows of X with streaming loads, so that a hub row's gathers are
-     * not kept in the L2 caches.  Pays only where the rows a hub gathers are not gathered again
-     * soon by other rows; results are unchanged. */
-    int32_t stream_rows_over;
     /* NNZ schedule, optional (NULL = the fix-up pass looks at every run): the rows that the
      * runs cut and the rows without entries, ascending, as numbers of stored rows.  With run
      * length K = cgnn_spmm_run_length(A), row r is cut when rowptr[r+1] - rowptr[r] > K and
@@ -122,8 +117,15 @@ int cgnn_spmm(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
  * cgnn_spmm_workspace_bytes exceeds that is refused with CGNN_EWORKSPACE (at F = 128 and the
  * default run length that is about 8 M non-zeros in the nnz schedule; the row schedule needs no
  * scratch and has no limit).  All calls on one GPU share the one array: calls that overlap
- * in time on the same GPU (two streams, two threads) race on it. */
+ * in time on the same GPU (two streams, two threads) race on it.
+ * cgnn_spmm_static_init() looks up the array's address on the device that is current in the
+ * calling thread (hipGetSymbolAddress, which may make the runtime load the library's device
+ * image there: not an operation a stream capture can record).  cgnn_spmm_static does the same on
+ * its first call on a device; a caller that captures, or that must not trigger the load inside
+ * its loop, calls cgnn_spmm_static_init once per device beforehand.  After that a call launches
+ * kernels and nothing else. */
 size_t cgnn_spmm_static_scratch_bytes(void);
+int cgnn_spmm_static_init(void);
 int cgnn_spmm_static(const cgnn_csr *A, int dtype, const void *X, void *Y, int64_t F,
                      int accumulate, int kernel, cgnn_stream_t stream);
 

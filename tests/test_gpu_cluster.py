@@ -272,3 +272,64 @@ def test_memory_probes_move_what_they_say():
     abi.check(L.cgnn_read_bytes(abi.ptr(src), ctypes.c_size_t(n), abi.ptr(sink), abi.stream_of(src)))
     torch.cuda.synchronize()
     assert L.cgnn_fill_bytes(abi.ptr(dst), ctypes.c_size_t(7), abi.stream_of(dst)) != 0
+
+
+def test_reference_signature_operators_read_the_host_once_per_index():
+    """The operators called with the reference's own argument lists (index and nothing else,
+    src/runtime/csrc/cluster/cluster_ops.h:5-13): the reference reads the host once per assignment
+    (cluster_kernel.cu:147) and never in mean / reconstruct.  Here the ids that cluster_assign
+    returned are known to the operators (no read at all), an index from elsewhere is checked on
+    its first use only, and an index that was written to since is checked again.  Host reads are
+    caught by torch's synchronisation check (any .item() / .cpu() of a device tensor raises)."""
+    import compressgnn_runtime as rt
+    rng = np.random.default_rng(4)
+    n, F, Fo, bits = 30000, 40, 24, 9
+    xn = rng.standard_normal((n, F)).astype(np.float32)
+    pl = rng.standard_normal((F, bits)).astype(np.float32)
+    x, planes = torch.from_numpy(xn).to(DEV), torch.from_numpy(pl).to(DEV)
+    ids, counts, active = rt.cluster_assign(x, planes, bits, rt.cluster_workspace(x, bits))
+    groups = active + 1
+    hidden = torch.from_numpy(rng.standard_normal((groups, Fo)).astype(np.float32)).to(DEV)
+    bias = torch.from_numpy(rng.standard_normal(Fo).astype(np.float32)).to(DEV)
+    go = torch.from_numpy(rng.standard_normal((n, Fo)).astype(np.float32)).to(DEV)
+    gr = torch.from_numpy(rng.standard_normal((groups, F)).astype(np.float32)).to(DEV)
+
+    def chain(index):
+        reps = rt.cluster_mean(x, index, counts)
+        out = rt.cluster_reconstruct(hidden, index, bias, True)
+        rg = rt.cluster_reconstruct_backward(go, index, out, groups, True)
+        dx = rt.cluster_mean_backward(gr, index, counts)
+        return reps, out, rg, dx
+
+    def without_host_reads(fn):
+        torch.cuda.synchronize()
+        torch.cuda.set_sync_debug_mode("error")
+        try:
+            return fn()
+        finally:
+            torch.cuda.set_sync_debug_mode("default")
+
+    # the check does catch a host read
+    with pytest.raises(RuntimeError):
+        without_host_reads(lambda: counts.sum().item())
+    got = without_host_reads(lambda: chain(ids))
+    ids_np, counts_np = ids.cpu().numpy(), counts.cpu().numpy()
+    want_reps = oracle.cluster_mean(xn, ids_np, counts_np)
+    want_out = oracle.reconstruct(hidden.cpu().numpy(), ids_np, bias.cpu().numpy(), True)
+    assert_within(got[0].cpu().numpy(), want_reps, rtol=1e-4, atol=1e-5)
+    assert np.array_equal(got[1].cpu().numpy(), want_out)
+    assert_within(got[2].cpu().numpy(), oracle.reconstruct_backward(go.cpu().numpy(), ids_np, want_out, groups, True), rtol=1e-4, atol=1e-5)
+    assert np.array_equal(got[3].cpu().numpy(), oracle.cluster_mean_backward(gr.cpu().numpy(), ids_np, counts_np))
+    # an index from elsewhere: checked on first use (gather first, then a reduction), silent afterwards
+    for first in (lambda i: rt.cluster_reconstruct(hidden, i, bias, True), lambda i: rt.cluster_mean(x, i, counts)):
+        foreign = ids.clone()
+        first(foreign)
+        again = without_host_reads(lambda: chain(foreign))
+        for a, b in zip(again, got):
+            assert torch.equal(a, b)
+        # written to since: no longer trusted, and the bad id is reported
+        foreign[17] = groups + 5
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_reconstruct(hidden, foreign, bias, True)
+        with pytest.raises(RuntimeError, match="outside"):
+            rt.cluster_mean(x, foreign, counts)

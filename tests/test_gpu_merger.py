@@ -1,7 +1,10 @@
-"""The batch compressor on the GPU (module compressgnn_batch_cuda) against the host
-compressor: the same arrays, as the reference's tests/test_batch_compression.py:52-59
-asks of its two backends, on the reference's grid of row shapes and on the graphs of the
-benchmark configurations."""
+"""The batch compressor on the GPU (module compressgnn_batch_cuda): its output is held to the
+contract the reference's tests pin at the compressor boundary -- int32 arrays, children below the
+rule's id, every vertex row expanding to exactly the input row in order
+(tests/test_batch_compression.py:15-36,52-55, tests/test_offline_compression.py:7-25), checked by
+a numpy expansion that shares no code with the product -- and, beside that, to the arrays of the
+host compressor (tests/test_batch_compression.py:52-59 asks that of the two backends), on the
+reference's grid of row shapes and on the graphs of the benchmark configurations."""
 import os
 import sys
 
@@ -12,6 +15,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "compressgnn_amd"))
 sys.path.insert(0, os.path.join(ROOT, "compressgnn_amd", "loader"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 pytestmark = pytest.mark.gpu
 
@@ -20,8 +24,9 @@ def both(v, e, rounds, freq):
     import compressgnn_batch_cuda as gpu
     from compressgnn_amd import compressgnn_offline as off
     want = off.compress_csr_batch(v, e, 4, rounds, freq)
+    from util import assert_compression_contract
     got = gpu.compress_csr_batch(v, e, rounds=rounds, min_pair_frequency=freq)
-    assert got[0].dtype == np.int32 and got[1].dtype == np.int32
+    assert_compression_contract(v, e, got)
     assert got[2] == want[2] and got[3] == want[3]
     assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
     return got

@@ -16,12 +16,13 @@ import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 for p in (ROOT, os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compressgnn_amd", "layer"),
-          os.path.join(ROOT, "compressgnn_amd", "loader")):
+          os.path.join(ROOT, "compressgnn_amd", "loader"), os.path.join(ROOT, "tests")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
 import oracle
 from compressgnn_amd import abi
+from util import assert_compression_contract, closed_form_transpose
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -355,6 +356,10 @@ def merger_case(rng, fail):
         v, e = off.add_self_loop_csr(v, e)
     want = off.compress_csr_batch(v, e, 4, rounds, freq)
     got = gpu.compress_csr_batch(v, e, rounds=rounds, min_pair_frequency=freq)
+    try:  # the reference's contract at this boundary, on the GPU's arrays directly
+        assert_compression_contract(v, e, got)
+    except AssertionError as exc:
+        return fail(params, "contract of the compressor boundary broken: %s" % exc)
     if not (got[2] == want[2] and got[3] == want[3] and np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])):
         fail(params, "%d rules on the GPU, %d on the host" % (got[3], want[3]))
 
@@ -378,10 +383,13 @@ def transpose_case(rng, fail):
         elist = np.concatenate([np.sort(elist[vlist[r]:vlist[r + 1]]) for r in range(rows)]
                                + [np.zeros(0, np.int64)]).astype(np.int64)
     value = rng.standard_normal(len(elist)).astype(np.float32)
-    want = off.csr_transpose(vlist, elist, value, cols)
+    want = closed_form_transpose(vlist, elist, value, cols)  # numpy's stable sort by column: no product code
     for a, w in zip(rt.csr_transpose(t(vlist), t(elist), t(value), cols), want):
         if not np.array_equal(a.cpu().numpy(), w):
-            return fail(params, "not the arrays of the host transpose")
+            return fail(params, "not the stable sort by column")
+    for a, w in zip(off.csr_transpose(vlist, elist, value, cols), want):
+        if not np.array_equal(a, w):
+            return fail(params, "host transpose: not the stable sort by column")
 
 
 def test_transposes():

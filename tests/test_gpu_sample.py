@@ -15,7 +15,7 @@ sys.path[:0] = [os.path.join(ROOT, "compressgnn_amd"), os.path.join(ROOT, "compr
                 os.path.join(ROOT, "compressgnn_amd", "loader")]
 
 import oracle
-from test_oracle_sample import GOLD, blocks_of, compressed, golden_blocks, misfit_graph
+from test_oracle_sample import GOLD, _chi2_ok, blocks_of, compressed, golden_blocks, misfit_graph, selection_law
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -135,6 +135,73 @@ def test_plain_form_and_large_fanouts():
     # positions are distinct: 3,000 of the hub's 6,000 distinct in-neighbours, no repeats
     samples, rows, cols = (x.cpu().numpy() for x in sampler.neighbor_sample_ori_impl(t(colptr), t(row), t(np.array([5])), [3000]))
     assert len(rows) == 3000 and len(set(samples[rows])) == 3000 and np.all(cols == 0)
+
+
+def test_sampled_positions_follow_the_law_of_the_reference_loop():
+    """The device sampler's own draws: over 8,000 frontier positions the in-neighbours of a vertex,
+    and the pairs of them, are taken with the frequencies the reference's selection loop has under
+    independent uniform draws (enumerated exactly, tests/test_oracle_sample.py), in the plain form
+    and through the rule hierarchy of a compressed graph; and the result is the oracle's."""
+    import compressgnn_sample as sampler
+    d, fan, n = 12, 5, 8000
+    single, pair = selection_law(d, fan)
+    iu = np.triu_indices(d, 1)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(DEV)
+
+    def held_to_the_law(picked, label):
+        assert all(len(set(p)) == fan for p in picked)
+        ok, stat = _chi2_ok(np.bincount(picked.ravel(), minlength=d), n * single)
+        assert ok, (label, "single", stat)
+        member = np.zeros((n, d), bool)
+        member[np.arange(n)[:, None], picked] = True
+        ok, stat = _chi2_ok((member[:, :, None] & member[:, None, :]).sum(0)[iu], n * pair[iu])
+        assert ok, (label, "pairs", stat)
+
+    colptr = np.array([0, d] + [d] * d, dtype=np.int64)
+    row = np.arange(1, d + 1, dtype=np.int64)
+    inp = np.zeros(n, np.int64)
+    got = [x.cpu().numpy() for x in sampler.neighbor_sample_ori_impl(t(colptr), t(row), t(inp), [fan], seed=21)]
+    want = oracle.neighbor_sample(dict(v2v=(colptr, row)), inp, [fan], seed=21, plain=True)
+    for a, w in zip(got, want):
+        assert np.array_equal(a, w)
+    held_to_the_law(got[0][got[1]].reshape(n, fan) - 1, "plain")
+    # a vertex of a compressed graph with 12 expanded in-neighbours: positions resolve through the rules
+    data, v, e = compressed("shared_lists")
+    b = blocks_of(data.edge_index)
+    node = 105
+    assert data.rule_cnt > 0 and int(b["v_degree"][node]) == d
+    assert b["v2r"][0][node + 1] > b["v2r"][0][node], "the vertex should be reached through rules"
+    full = oracle.neighbor_list(b, node)
+    assert sorted(full.tolist()) == list(range(11)) + [node]
+    inp = np.full(n, node, np.int64)
+    got = [x.cpu().numpy() for x in sampler.neighbor_sample_cg_sim(*on_device(b), t(inp), [fan], seed=22)]
+    want = oracle.neighbor_sample(b, inp, [fan], seed=22)
+    for a, w in zip(got, want):
+        assert np.array_equal(a, w)
+    # neighbour -> its position in get_neighbor's numbering
+    by_position = oracle.get_neighbors(b, np.full(d, node, np.int64), np.arange(d, dtype=np.int64))
+    position_of = {int(x): k for k, x in enumerate(by_position)}
+    picked = np.array([position_of[int(x)] for x in got[0][got[2]]]).reshape(n, fan)
+    held_to_the_law(picked, "compressed")
+
+
+def test_oversized_fanout_is_refused_not_truncated():
+    """A fan-out of 2^31 or more below the degree of a vertex cannot be a count of this layer:
+    the call fails (the status the kernels raise), it does not sample fanout mod 2^32."""
+    import compressgnn_sample as sampler
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(DEV)
+    colptr = np.array([0, 3, 3, 3, 3], dtype=np.int64)
+    row = np.array([1, 2, 3], dtype=np.int64)
+    # degree 3 <= fan-out: the full list, whatever the size of the fan-out
+    samples, rows, cols = sampler.neighbor_sample_ori_impl(t(colptr), t(row), t(np.array([0])), [2 ** 40])
+    assert samples.cpu().tolist() == [0, 1, 2, 3]
+    data, v, e = compressed("blocks")
+    b = blocks_of(data.edge_index)
+    huge = dict(b)
+    huge["v_degree"] = np.asarray(b["v_degree"]).copy()
+    huge["v_degree"][0] = 2 ** 33  # claims more neighbours than any fan-out below
+    with pytest.raises((RuntimeError, IndexError)):
+        sampler.neighbor_sample_cg_sim(*on_device(huge), t(np.array([0])), [2 ** 32 + 1])
 
 
 def test_sampler_errors():

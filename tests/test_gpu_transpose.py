@@ -1,5 +1,6 @@
-"""The on-GPU CSR -> CSC transpose against the host library's (bit for bit: the order is
-the one SparseTensor.csc() gives -- by column, ties in storage order)."""
+"""The on-GPU CSR -> CSC transpose against the order mathematics fixes (a stable sort of the
+entries by column: what SparseTensor.csc() gives, reference layer/CompressgnnSPMM.py:68-70),
+computed here with numpy alone, and against the host library's transpose beside it."""
 import os
 import sys
 
@@ -11,6 +12,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "compressgnn_amd"))
 sys.path.insert(0, os.path.join(ROOT, "compressgnn_amd", "loader"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -40,7 +42,10 @@ def test_device_transpose_matches_host(rows, cols, mean, dup):
     from compressgnn_amd import compressgnn_offline as off
     rng = np.random.default_rng(rows * 7 + cols)
     vlist, elist, value = random_block(rng, rows, cols, mean, dup)
-    want = off.csr_transpose(vlist, elist, value, cols)
+    from util import closed_form_transpose
+    want = closed_form_transpose(vlist, elist, value, cols)
+    for a, b in zip(off.csr_transpose(vlist, elist, value, cols), want):  # the host routine, beside it
+        assert np.array_equal(a, b)
     t = lambda a: torch.from_numpy(a).to(DEV)
     for impl in (rt.csr_transpose, abi.csr_transpose):
         colptr, row, tval = impl(t(vlist), t(elist), t(value), cols)
@@ -80,7 +85,8 @@ def test_sparse_block_transposes_where_it_lives():
     host = SparseCSR(torch.from_numpy(vlist), torch.from_numpy(elist), torch.from_numpy(value), (900, 700))
     dev = host.to(DEV)
     assert dev._csc is None
-    for a, b in zip(host.csc(), dev.csc()):
-        assert b.device.type == "cuda" and torch.equal(a, b.cpu())
+    from util import closed_form_transpose
+    for a, b, c in zip(host.csc(), dev.csc(), closed_form_transpose(vlist, elist, value, 700)):
+        assert b.device.type == "cuda" and torch.equal(a, b.cpu()) and np.array_equal(b.cpu().numpy(), c)
     tt = dev.t()
     assert tt.sparse_sizes() == (700, 900) and torch.equal(tt.csr()[1].cpu(), host.csc()[1])

@@ -270,3 +270,27 @@ def test_offloaded_blocks_deliver_to_their_device():
     assert not g.offloaded and g.device.type == "cpu"
     assert all(torch.equal(a, b) for a, b in zip(g.csr(), before))
     assert all(torch.equal(a, b) for a, b in zip(g.csc(), csc_before))
+
+
+def test_host_merger_and_transpose_meet_the_independent_checkers():
+    """The numpy checkers the GPU tests hold the device routines to (tests/util.py), applied to
+    the host routines: the contract of the compressor boundary and the stable sort by column."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from util import assert_compression_contract, closed_form_transpose
+    rng = np.random.default_rng(9)
+    for V, freq in ((1, 3), (300, 3), (6000, 8)):
+        v, e = (off.gen_copy_model(V, 9.8, 0.7, 5) if V > 1 else (np.array([0, 0], np.int64), np.zeros(0, np.int64)))
+        got = off.compress_csr_batch(v, e, 4, 12, freq)
+        assert_compression_contract(v, e, got)
+        if got[3]:
+            broken = got[1].copy()
+            broken[0] = (broken[0] + 1) % V
+            with pytest.raises(AssertionError):
+                assert_compression_contract(v, e, (got[0], broken, got[2], got[3]))
+    for rows, cols in ((7, 3), (300, 500), (5000, 300)):
+        lens = rng.poisson(4, rows)
+        v = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        e = rng.integers(0, cols, int(v[-1])).astype(np.int64)
+        val = rng.standard_normal(len(e)).astype(np.float32)
+        for a, b in zip(off.csr_transpose(v, e, val, cols), closed_form_transpose(v, e, val, cols)):
+            assert np.array_equal(a, b)

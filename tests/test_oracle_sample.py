@@ -54,6 +54,14 @@ def compressed(kind, seed=3):
         n = 64
         v = np.arange(n + 1, dtype=np.int64) * 32
         e = np.tile(np.arange(32, dtype=np.int64), n)
+    elif kind == "shared_lists":
+        # 11 vertices with the same 32 targets: every target has 11 in-neighbours that are reached
+        # through rules, and itself (the self loop)
+        V = 140
+        lens = np.zeros(V, np.int64)
+        lens[:11] = 32
+        v = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        e = np.tile(np.arange(100, 132, dtype=np.int64), 11)
     elif kind == "copy":
         v, e = off.gen_copy_model(1500, 9.0, 0.7, seed)
     else:
@@ -209,3 +217,95 @@ def test_selection_loop_properties():
     draws = [oracle.counter_draw(5, 1, 10, j, j) for j in range(1, 200)]
     assert all(0 <= d < j for d, j in zip(draws, range(1, 200)))
     assert len(set(oracle.counter_draw(5, 1, i, 1000, 1000) for i in range(100))) > 60
+
+
+def _chi2_ok(observed, expected, alpha=1e-6):
+    """Pearson's statistic against the 1 - alpha quantile: a sound generator fails once in a million runs
+    (the draws are a fixed function of fixed seeds, so the outcome is the same on every run)."""
+    from scipy.stats import chi2
+    observed, expected = np.asarray(observed, float).ravel(), np.asarray(expected, float).ravel()
+    stat = float(((observed - expected) ** 2 / expected).sum())
+    return stat < chi2.ppf(1 - alpha, len(observed) - 1), stat
+
+
+def test_counter_draws_are_uniform_and_independent():
+    """What mathematics fixes about the counter-based generator (the reference draws uniformly from
+    [0, high) with a sequential generator, src/sample/csrc/neighbor_sample.h:10-15,112-118; a
+    parallel sampler cannot replay that stream, but its draws must have the same law): every draw
+    uniform over its range, and draws that differ in one key only (frontier position, step, layer,
+    seed) independent of each other.  A biased multiply-high, a counter that ignores a key or two
+    keys that collapse into one would each fail here."""
+    n = 30000
+    draw = oracle.counter_draw
+    for high in (2, 3, 7, 10, 64, 1000, 12345, 2 ** 31 - 1, 2 ** 40 + 7):
+        d = np.array([draw(11, 0, i, high, high) for i in range(n)], dtype=np.float64)
+        assert d.min() >= 0 and d.max() < high
+        bins = min(high, 50)
+        counts = np.bincount((d * bins / high).astype(np.int64), minlength=bins)
+        edges = np.floor(np.arange(bins + 1) * high / bins + 0.999999) if high > bins else np.arange(bins + 1)
+        expected = n * np.diff(edges) / high if high > bins else np.full(bins, n / bins)
+        ok, stat = _chi2_ok(counts, expected)
+        assert ok, ("marginal", high, stat)
+    high = 6
+    base = np.array([draw(11, 0, i, 9, high) for i in range(n)])
+    variants = {
+        "next position": np.array([draw(11, 0, i + 1, 9, high) for i in range(n)]),
+        "next step": np.array([draw(11, 0, i, 10, high) for i in range(n)]),
+        "next layer": np.array([draw(11, 1, i, 9, high) for i in range(n)]),
+        "next seed": np.array([draw(12, 0, i, 9, high) for i in range(n)]),
+        "position and step exchanged": np.array([draw(11, 0, 9, i, high) for i in range(n)]),
+    }
+    for name, other in variants.items():
+        joint = np.bincount(base * high + other, minlength=high * high)
+        ok, stat = _chi2_ok(joint, np.full(high * high, n / (high * high)))
+        assert ok, (name, stat)
+        assert np.count_nonzero(base != other) > n // 2, name
+    # steps of one vertex (the selection loop walks j upwards with high = j): no drift along j
+    u = np.array([draw(3, 2, 77, j, j) / j for j in range(1, n + 1)])
+    ok, stat = _chi2_ok(np.bincount((u[100:] * 20).astype(np.int64), minlength=20), np.full(20, (n - 100) / 20))
+    assert ok, ("along the steps", stat)
+
+
+def selection_law(d, fan):
+    """Exact inclusion probabilities (single positions, pairs) of the reference's selection loop
+    under independent uniform draws, by enumerating every draw sequence."""
+    import itertools
+    single, pair, total = np.zeros(d), np.zeros((d, d)), 0
+    for draws in itertools.product(*[range(j) for j in range(d - fan, d)]):
+        chosen = []
+        for j, rnd in zip(range(d - fan, d), draws):
+            chosen.append(j if rnd in chosen else rnd)
+        single[chosen] += 1
+        for a in chosen:
+            pair[a, chosen] += 1
+        total += 1
+    return single / total, pair / total
+
+
+def test_selection_loop_follows_the_law_of_the_reference_loop():
+    """The selection loop (neighbor_sample.h:112-118) fed by the counter-based generator.  The loop
+    draws step j from [0, j), j excluded (torch::randint's upper bound, :10-15), and takes j itself on a
+    collision, so the positions are not equally likely (the last one is taken on a collision
+    only).  Its exact law under independent uniform draws is enumerated here -- all 7*8*9*10*11
+    draw sequences for 5 of 12 -- and the frequencies of single positions and of pairs over many
+    frontier positions are held to it."""
+    d, fan, n = 12, 5, 8000
+    single, pair = selection_law(d, fan)
+    assert abs(single.sum() - fan) < 1e-9 and single[d - 1] < single[0]
+    colptr = np.array([0, d] + [d] * d, dtype=np.int64)
+    row = np.arange(1, d + 1, dtype=np.int64)
+    samples, rows, cols = oracle.neighbor_sample(dict(v2v=(colptr, row)), np.zeros(n, np.int64), [fan], seed=5, plain=True)
+    assert len(rows) == n * fan
+    picked = samples[rows].reshape(n, fan) - 1  # plain form: rows index the sampled neighbours
+    assert all(len(set(p)) == fan for p in picked)
+    ok, stat = _chi2_ok(np.bincount(picked.ravel(), minlength=d), n * single)
+    assert ok, ("single", stat)
+    member = np.zeros((n, d), bool)
+    member[np.arange(n)[:, None], picked] = True
+    iu = np.triu_indices(d, 1)
+    seen = (member[:, :, None] & member[:, None, :]).sum(0)[iu]
+    ok, stat = _chi2_ok(seen, n * pair[iu])
+    assert ok, ("pairs", stat)
+    # the uniform law would be rejected by the same data: the test can tell the two apart
+    ok, stat = _chi2_ok(np.bincount(picked.ravel(), minlength=d), np.full(d, n * fan / d))
+    assert not ok

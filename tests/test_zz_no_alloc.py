@@ -77,3 +77,22 @@ def test_static_scratch_refuses_what_does_not_fit():
                             abi.stream_of(rowptr))
     assert rc == 2 and b"built-in" in L.cgnn_last_error()  # CGNN_EWORKSPACE
     torch.cuda.synchronize()
+
+
+def test_static_entry_leaves_device_memory_as_it_found_it():
+    """'Allocates nothing', measured: once the array's address is known on the device
+    (cgnn_spmm_static_init, outside any capture), calls leave the free memory of the device where
+    it was -- the driver's own figure (hipMemGetInfo), which no caching allocator hides."""
+    assert abi.lib().cgnn_spmm_static_init() == 0
+    A, X, Y0 = _case(3, 20000, 15000, 128, giant=200_000)
+    Y = torch.empty_like(Y0)
+    abi.spmm_static(A, X, Y, False, abi.SPMM_NNZ)  # warmed: kernels loaded
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for kernel in (abi.SPMM_NNZ, abi.SPMM_ROW, abi.SPMM_AUTO):
+        abi.spmm_static(A, X, Y, False, kernel)
+        abi.spmm_static(A, X, Y, True, kernel)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    assert torch.equal(abi.spmm_static(A, X, Y, False, abi.SPMM_NNZ), abi.spmm(A, X, None, False, abi.SPMM_NNZ))

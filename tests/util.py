@@ -56,3 +56,61 @@ def assert_no_less_accurate(got, sequential, truth, factor=2.0):
     print("accuracy vs float64: kernel max %.3e mean %.3e | sequential fp32 max %.3e mean %.3e" % (
         e_got.max(), e_got.mean(), e_seq.max(), e_seq.mean()))
     return float(e_got.max()), float(e_seq.max())
+
+
+def closed_form_transpose(vlist, elist, value, cols):
+    """CSR -> CSC as mathematics fixes it: a stable sort of the entries by column (ties keep
+    storage order, which is what SparseTensor.csc() gives).  No product code involved."""
+    vlist, elist = np.asarray(vlist, np.int64), np.asarray(elist, np.int64)
+    order = np.argsort(elist, kind="stable")
+    rowidx = np.repeat(np.arange(len(vlist) - 1, dtype=np.int64), np.diff(vlist))
+    colptr = np.concatenate([[0], np.cumsum(np.bincount(elist, minlength=cols))]).astype(np.int64)
+    return colptr, rowidx[order], (None if value is None else np.asarray(value)[order])
+
+
+def expand_compressed_rows(out_ptr, out_col, V):
+    """The vertex rows of a compressed CSR (rows V.. are rules) with every rule replaced by its
+    children, recursively, in place and in order.  Returns (rowptr, columns) of the expansion."""
+    out_ptr, out_col = np.asarray(out_ptr, np.int64), np.asarray(out_col, np.int64)
+    rule_ptr = out_ptr[V:] - out_ptr[V]
+    rule_col = out_col[out_ptr[V]:]
+    rule_len = np.diff(rule_ptr)
+    col = out_col[:out_ptr[V]].copy()
+    row = np.repeat(np.arange(V, dtype=np.int64), np.diff(out_ptr[:V + 1]))
+    for _ in range(64):
+        is_rule = col >= V
+        if not is_rule.any():
+            break
+        lens = np.where(is_rule, rule_len[np.where(is_rule, col - V, 0)], 1)
+        start = np.concatenate([[0], np.cumsum(lens)])
+        new_row = np.repeat(row, lens)
+        within = np.arange(start[-1]) - np.repeat(start[:-1], lens)
+        src_rule = np.repeat(np.where(is_rule, col - V, 0), lens)
+        from_rule = np.repeat(is_rule, lens)
+        new_col = np.where(from_rule, rule_col[np.minimum(rule_ptr[src_rule] + within, max(len(rule_col) - 1, 0))]
+                           if len(rule_col) else 0, np.repeat(col, lens))
+        col, row = new_col, new_row
+    else:
+        raise AssertionError("rules nest deeper than 64 levels (a cycle?)")
+    rowptr = np.concatenate([[0], np.cumsum(np.bincount(row, minlength=V))]).astype(np.int64)
+    return rowptr, col
+
+
+def assert_compression_contract(vlist, elist, got):
+    """What the reference's tests pin at the compressor boundary
+    (tests/test_batch_compression.py:15-36,52-55, tests/test_offline_compression.py:7-25): int32
+    arrays, a well-formed CSR over V + R rows, every child of a rule has a smaller id than the
+    rule, and every vertex row expands to exactly the input row, in order."""
+    out_ptr, out_col, V, R = got
+    vlist, elist = np.asarray(vlist, np.int64), np.asarray(elist, np.int64)
+    assert out_ptr.dtype == np.int32 and out_col.dtype == np.int32
+    assert V == len(vlist) - 1 and len(out_ptr) == V + R + 1
+    assert out_ptr[0] == 0 and out_ptr[-1] == len(out_col) and (np.diff(out_ptr) >= 0).all()
+    if len(out_col):
+        assert out_col.min() >= 0 and out_col.max() < V + R
+    if R:
+        rule_rows = np.repeat(np.arange(V, V + R), np.diff(out_ptr[V:]))
+        assert (out_col[out_ptr[V]:] < rule_rows).all(), "a rule refers to itself or to a later rule"
+        assert (np.diff(out_ptr[V:]) >= 2).all(), "a rule with fewer than two children"
+    rowptr, col = expand_compressed_rows(out_ptr, out_col, V)
+    assert np.array_equal(rowptr, vlist - vlist[0]) and np.array_equal(col, elist)
