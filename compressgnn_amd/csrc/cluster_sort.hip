@@ -16,6 +16,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "radix_sort.h"
 
 namespace cgnn {
 namespace {
@@ -456,6 +457,15 @@ struct GroupLayout {
 };
 
 }  // namespace
+
+// The sort for the rest of the library (radix_sort.h).
+size_t radix_sort_counter_bytes(int64_t N) { return radix_counter_bytes(N); }
+
+int radix_sort_positions(const int32_t *keys, int64_t N, int bits, int32_t *keys_out, int32_t *pos_out,
+                         int32_t *tmp_keys, int32_t *tmp_pos, void *counters, hipStream_t stream) {
+    return radix_sort_by_key(keys, N, bits, keys_out, pos_out, tmp_keys, tmp_pos, counters, nullptr, 0, nullptr, nullptr,
+                             stream);
+}
 
 size_t occupancy_scan_bytes(int64_t n);
 int occupancy_scan(const int32_t *in, int64_t n, int32_t *out, void *scratch, hipStream_t stream);

@@ -2,14 +2,14 @@
 // layer/CompressgnnSPMM.py:68-70, loader/compress_graph.py:21-35 rely on it): entries
 // sorted by column, ties in storage order, i.e. by row and then by position in the row.
 //
-// The entries are numbered in storage order and sorted by column with rocPRIM's stable
-// LSD radix sort (through hipCUB), limited to the bits the column numbers occupy; the
-// sorted position p then takes the row and value of entry perm[p], and colptr[c] is the
-// first sorted position whose column is >= c.  Nothing here depends on timing: the result
-// is the same array, bit for bit, as the host routine cgnn_csr_transpose produces.
-#include <hipcub/hipcub.hpp>
-
+// The entries are numbered in storage order and sorted by column with the library's own
+// stable LSD radix sort (radix_sort.h; the payload of a key is its position), limited to the
+// bits the column numbers occupy; the sorted position p then takes the row and value of
+// entry perm[p], and colptr[c] is the first sorted position whose column is >= c.  Nothing
+// here depends on timing: the result is the same array, bit for bit, as the host routine
+// cgnn_csr_transpose produces.
 #include "common.h"
+#include "radix_sort.h"
 
 namespace cgnn {
 namespace {
@@ -17,32 +17,26 @@ namespace {
 constexpr int64_t kTransposeLimit = (int64_t)INT32_MAX - 65536;
 
 struct TransposeWorkspace {
-    size_t keys_in, keys_out, pos_in, pos_out, sort_temp, total;
+    size_t keys_in, keys_out, pos_out, tmp_keys, tmp_pos, counters, total;
 };
-
-size_t transpose_sort_temp(int64_t nnz) {
-    size_t bytes = 0;
-    hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
-                                       (const uint32_t *)nullptr, (uint32_t *)nullptr, (int)nnz, 0, 32, 0);
-    return bytes;
-}
 
 TransposeWorkspace transpose_workspace(int64_t nnz) {
     TransposeWorkspace w{};
-    const size_t arr = align_up((size_t)nnz * sizeof(uint32_t), 256);
+    const size_t arr = align_up((size_t)nnz * sizeof(int32_t), 256);
     w.keys_in = 0;
     w.keys_out = arr;
-    w.pos_in = 2 * arr;
-    w.pos_out = 3 * arr;
-    w.sort_temp = 4 * arr;
-    w.total = 4 * arr + align_up(transpose_sort_temp(nnz), 256);
+    w.pos_out = 2 * arr;
+    w.tmp_keys = 3 * arr;
+    w.tmp_pos = 4 * arr;
+    w.counters = 5 * arr;
+    w.total = 5 * arr + align_up(radix_sort_counter_bytes(nnz), 256);
     return w;
 }
 
-// keys[e] = column of entry e, pos[e] = e; flag is raised for a column outside [0, cols).
+// keys[e] = column of entry e (the sort numbers the entries itself); flag is raised for a
+// column outside [0, cols).
 __global__ void transpose_keys_kernel(const int64_t *__restrict__ col, int64_t nnz, int64_t cols,
-                                      uint32_t *__restrict__ keys, uint32_t *__restrict__ pos,
-                                      int32_t *__restrict__ bad) {
+                                      int32_t *__restrict__ keys, int32_t *__restrict__ bad) {
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz;
          e += (int64_t)gridDim.x * blockDim.x) {
         const int64_t c = col[e];
@@ -50,16 +44,15 @@ __global__ void transpose_keys_kernel(const int64_t *__restrict__ col, int64_t n
             *bad = 1;  // every writer stores the same value
             keys[e] = 0;
         } else {
-            keys[e] = (uint32_t)c;
+            keys[e] = (int32_t)c;
         }
-        pos[e] = (uint32_t)e;
     }
 }
 
 // Row and value (a 4- or 8-byte word W) of the entry that lands at sorted position p.
 template <typename W>
 __global__ void transpose_fill_kernel(const int64_t *__restrict__ rowptr, int64_t rows, int64_t nnz,
-                                      const uint32_t *__restrict__ perm, const W *__restrict__ val,
+                                      const int32_t *__restrict__ perm, const W *__restrict__ val,
                                       int64_t *__restrict__ row_out, W *__restrict__ val_out) {
     for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < nnz;
          p += (int64_t)gridDim.x * blockDim.x) {
@@ -76,7 +69,7 @@ __global__ void transpose_fill_kernel(const int64_t *__restrict__ rowptr, int64_
 }
 
 // colptr[c] = first sorted position whose column is >= c, for c = 0..cols.
-__global__ void transpose_colptr_kernel(const uint32_t *__restrict__ sorted_col, int64_t nnz, int64_t cols,
+__global__ void transpose_colptr_kernel(const int32_t *__restrict__ sorted_col, int64_t nnz, int64_t cols,
                                         int64_t *__restrict__ colptr) {
     for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c <= cols;
          c += (int64_t)gridDim.x * blockDim.x) {
@@ -121,7 +114,7 @@ extern "C" int cgnn_csr_transpose_device(int64_t rows, int64_t cols, int64_t nnz
     hipLaunchKernelGGL(transpose_clear_flag_kernel, dim3(1), dim3(1), 0, stream, bad_column);
     if (nnz == 0) {
         hipLaunchKernelGGL(transpose_colptr_kernel, dim3(transpose_grid(cols + 1)), dim3(kBlock), 0, stream,
-                           (const uint32_t *)nullptr, (int64_t)0, cols, colptr_out);
+                           (const int32_t *)nullptr, (int64_t)0, cols, colptr_out);
         return check_launch("csr_transpose_device");
     }
     const TransposeWorkspace w = transpose_workspace(nnz);
@@ -130,21 +123,15 @@ extern "C" int cgnn_csr_transpose_device(int64_t rows, int64_t cols, int64_t nnz
         return CGNN_EWORKSPACE;
     }
     char *base = static_cast<char *>(workspace);
-    uint32_t *keys_in = reinterpret_cast<uint32_t *>(base + w.keys_in);
-    uint32_t *keys_out = reinterpret_cast<uint32_t *>(base + w.keys_out);
-    uint32_t *pos_in = reinterpret_cast<uint32_t *>(base + w.pos_in);
-    uint32_t *pos_out = reinterpret_cast<uint32_t *>(base + w.pos_out);
+    auto at = [&](size_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    int32_t *keys_in = at(w.keys_in), *keys_out = at(w.keys_out), *pos_out = at(w.pos_out);
     hipLaunchKernelGGL(transpose_keys_kernel, dim3(transpose_grid(nnz)), dim3(kBlock), 0, stream, col, nnz, cols,
-                       keys_in, pos_in, bad_column);
+                       keys_in, bad_column);
     int bits = 1;
-    while (bits < 32 && ((int64_t)1 << bits) < cols) ++bits;
-    size_t temp_bytes = workspace_bytes - w.sort_temp;
-    const hipError_t e = hipcub::DeviceRadixSort::SortPairs(base + w.sort_temp, temp_bytes, keys_in, keys_out, pos_in, pos_out,
-                                           (int)nnz, 0, bits, stream);
-    if (e != hipSuccess) {
-        set_error("cgnn_csr_transpose_device: sort failed: %s", hipGetErrorString(e));
-        return CGNN_ELAUNCH;
-    }
+    while (bits < 31 && ((int64_t)1 << bits) < cols) ++bits;
+    const int rc = radix_sort_positions(keys_in, nnz, bits, keys_out, pos_out, at(w.tmp_keys), at(w.tmp_pos),
+                                        base + w.counters, stream);
+    if (rc != CGNN_OK) return rc;
     if (dtype == CGNN_F64)
         hipLaunchKernelGGL(transpose_fill_kernel<uint64_t>, dim3(transpose_grid(nnz)), dim3(kBlock), 0, stream, rowptr,
                            rows, nnz, pos_out, static_cast<const uint64_t *>(val), row_out,
