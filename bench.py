@@ -329,6 +329,88 @@ def cpu_cluster_baseline(x, planes, detail, sample=200000):
 C4_VERTICES, C4_AVG_DEGREE, C4_F, C4_HIDDEN, C4_CLASSES, C4_H = 18_500_000, 16.1, 64, 64, 16, 16
 
 
+def c4_sampled_in_lists(off, v, e, vertices, hubs=8, others=3000):
+    """(vertices to check, and for every edge into one of them: source, position of the target among
+    the checked vertices, weight) from the uncompressed graph with self loops and symmetric
+    normalisation -- what the propagation must reproduce (loader/origin_data.py:10-82 of the
+    reference defines the uncompressed product the same way)."""
+    v2, e2 = off.add_self_loop_csr(v, e)
+    d = off.get_norm_degree(e2, vertices)
+    indeg = np.bincount(e2, minlength=vertices)
+    rng = np.random.default_rng(5)
+    checked = np.unique(np.concatenate([np.argsort(indeg)[-hubs:], rng.integers(0, vertices, others)]))
+    where = np.full(vertices, -1, np.int64)
+    where[checked] = np.arange(len(checked))
+    hit = np.nonzero(where[e2] >= 0)[0]
+    src = np.searchsorted(v2, hit, side="right") - 1
+    tgt = e2[hit]
+    w = (d[src] * d[tgt]).astype(np.float32)  # the weight of the uncompressed edge, in float32 as the loader has it
+    return checked, src.astype(np.int64), where[tgt], w, int(indeg[checked].max())
+
+
+def c4_check_propagation(torch, plan, x, sampled, detail):
+    """The propagation of the full-size graph against what no kernel of the library computes: float64
+    sums over the in-lists of sampled vertices (the most popular ones among them) taken from the
+    uncompressed graph, and the adjoint identity <A x, g> = <x, A^T g> over the whole tensors."""
+    checked, src, at, w, longest = sampled
+    dev = x.device
+    out = plan.forward(x)
+    ref = torch.zeros(len(checked), x.size(1), dtype=torch.float64, device=dev)
+    for lo in range(0, len(src), 1 << 22):
+        s = torch.from_numpy(src[lo:lo + (1 << 22)]).to(dev)
+        a = torch.from_numpy(at[lo:lo + (1 << 22)]).to(dev)
+        ww = torch.from_numpy(w[lo:lo + (1 << 22)]).to(dev).double()
+        ref.index_add_(0, a, x.index_select(0, s).double() * ww.unsqueeze(1))
+    got = out.index_select(0, torch.from_numpy(checked).to(dev)).double()
+    err = (got - ref).abs()
+    worst = float(err.max())
+    bad = int((err > 1e-6 + 1e-5 * ref.abs()).sum())
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    g = torch.randn(x.shape, device=dev, generator=gen)
+    gx = plan.backward(g)
+    lhs = float((out.double() * g.double()).sum())
+    rhs = float((x.double() * gx.double()).sum())
+    scale = float(out.double().norm() * g.double().norm())
+    detail["checks"] = dict(propagation_vertices_checked=int(len(checked)), longest_in_list_checked=longest,
+                            propagation_max_abs_err_vs_float64=worst, propagation_elements_outside_tolerance=bad,
+                            adjoint_lhs=lhs, adjoint_rhs=rhs, adjoint_relative_gap=abs(lhs - rhs) / scale)
+    if bad or not np.isfinite(worst):
+        raise RuntimeError("C4: propagation differs from the float64 sums over the uncompressed in-lists at %d elements "
+                           "(largest difference %.3g)" % (bad, worst))
+    if not abs(lhs - rhs) <= 1e-6 * scale:
+        raise RuntimeError("C4: <A x, g> = %.9g but <x, A^T g> = %.9g" % (lhs, rhs))
+
+
+def c4_check_clusters(torch, layers, inputs, detail):
+    """The assignments of the last epoch at full size: dense ids 1..active that all occur, sizes that
+    add up to the number of vertices, and the representatives of the largest and of 63 other
+    clusters against float64 means over their members (found by comparing ids, not through the
+    member lists of the library)."""
+    import compressgnn_runtime as rt
+    report = []
+    for layer, feats in zip(layers, inputs):
+        index, active = layer.cluster.vertex_index, int(layer.cluster.active_bucket)
+        N = index.numel()
+        sizes = torch.bincount(index, minlength=active + 1)
+        ok = (int(index.min()) >= 1 and int(index.max()) == active and int(sizes[0]) == 0 and int((sizes[1:] == 0).sum()) == 0
+              and int(sizes.sum()) == N and sizes.numel() == active + 1)
+        if not ok:
+            raise RuntimeError("C4: cluster ids are not the dense ids 1..%d of %d vertices" % (active, N))
+        reps = rt.cluster_mean(feats, index, sizes.to(torch.int32))
+        pick = torch.unique(torch.cat([sizes.argmax().view(1), torch.randint(1, active + 1, (63,), device=index.device)]))
+        worst = 0.0
+        for c in pick.tolist():
+            members = (index == c).nonzero().flatten()
+            mean = feats.index_select(0, members).double().mean(0)
+            worst = max(worst, float((reps[c].double() - mean).abs().max()))
+        report.append(dict(active=active, largest_cluster=int(sizes.max()), clusters_checked=int(pick.numel()),
+                           mean_max_abs_err_vs_float64=worst))
+        if not worst <= 1e-4:
+            raise RuntimeError("C4: cluster means differ from float64 means over the members by %.3g" % worst)
+    detail["checks"]["clusters"] = report
+
+
 def bench_c4(torch, vertices, epochs, refresh_interval):
     """C4: one training epoch of a 2-layer GCN whose layers are propagate -> cluster ->
     Linear on the representatives -> reconstruct(bias) (the layer of the reference's
@@ -348,6 +430,9 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
     v, e = off.gen_copy_model(vertices, C4_AVG_DEGREE, C1_COPY_PROB, C1_SEED)
     times["generate_s"] = time.time() - t0
     log("[bench] C4 graph generated: V=%d E=%d (%.1fs)" % (vertices, len(e), times["generate_s"]))
+    t0 = time.time()
+    sampled = c4_sampled_in_lists(off, v, e, vertices)
+    times["in_lists_for_the_check_s"] = time.time() - t0
     t0 = time.time()
     mask = np.ones(1, dtype=bool)  # masks are not used: the loss runs over all vertices
     data = CompressgnnData(np.zeros((vertices, 1), np.float32), (v, e), np.zeros(1, np.int64), mask, mask, mask,
@@ -386,6 +471,13 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
     gen.manual_seed(7)
     x = torch.randn(vertices, C4_F, device=dev, generator=gen)
     y = torch.randint(0, C4_CLASSES, (vertices,), device=dev, generator=gen)
+    # not timed, and before the peak-memory count starts: the propagation of this graph against
+    # float64 sums over the uncompressed in-lists and the adjoint identity
+    checks = {}
+    c4_check_propagation(torch, graph.plan(), x, sampled, checks)
+    del sampled
+    torch.cuda.empty_cache()
+    log("[bench] C4 propagation checked: %s" % json.dumps(checks["checks"]))
     torch.cuda.reset_peak_memory_stats()
 
     def epoch(k):
@@ -408,6 +500,15 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
         log("[bench] C4 epoch %d: %.1f ms, loss %.4f" % (k, ms[-1], losses[-1]))
     timed = ms[1:]
     refreshed = [layers[0].cluster.refresh_count, layers[1].cluster.refresh_count]
+    peak = int(torch.cuda.max_memory_allocated())
+    with torch.no_grad():  # the inputs of the two cluster layers, recomputed outside the timed epochs
+        p0 = layers[0].P(x=x, edge_index=graph, edge_weight=None, vertex_cnt=data.vertex_cnt, rule_cnt=data.rule_cnt)
+        h = layers[0](x, epochs).relu()
+        p1 = layers[1].P(x=h, edge_index=graph, edge_weight=None, vertex_cnt=data.vertex_cnt, rule_cnt=data.rule_cnt)
+        if refresh_interval == 1:  # the assignments held are those of these very inputs
+            layers[1](h, epochs)
+            c4_check_clusters(torch, layers, (p0, p1), checks)
+        del p0, p1, h
     return {
         "metric": "gcn_2layer_epoch_ms_C4", "value": float(np.mean(timed)), "unit": "ms", "n_gpus": 1,
         "steps": epochs, "warmup": 1, "ms_per_step": float(np.mean(timed)), "higher_is_better": False,
@@ -418,7 +519,7 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
                                                                    C4_H, refresh_interval),
                    "rules": int(data.rule_cnt), "compressed_edges": int(data.edge_cnt), "levels": int(graph.step)},
         "detail": {"epoch_ms": ms, "loss": losses, "cluster_refreshes": refreshed,
-                   "peak_hbm_bytes": int(torch.cuda.max_memory_allocated()),
+                   "peak_hbm_bytes": peak, "checks": checks["checks"],
                    "active_clusters": [int(layers[0].cluster.active_bucket), int(layers[1].cluster.active_bucket)],
                    "host_seconds": times},
     }
