@@ -65,6 +65,7 @@ struct DeviceCsr {
     int64_t rows = 0, cols = 0, nnz = 0;
     Tensor rowptr, colidx, rowidx, val;
     Tensor rowmap;  // optional: stored row g is output row rowmap[g]
+    int64_t out_rows = 0;  // rows of the output: `rows`, or more when only the rows with entries are stored (rule levels)
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
     Tensor cut_rows, empty_rows;  // the rows the runs of the nnz schedule cut / the rows without entries
@@ -133,11 +134,15 @@ struct DeviceCsr {
 // rowptr/col: int64 or int32 tensors on any device; value: float tensor or undefined.
 std::shared_ptr<DeviceCsr> make_csr(Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows,
                                     int64_t cols, torch::Device device, int64_t seg_nnz,
-                                    c10::optional<Tensor> rowmap = c10::nullopt, bool with_row_lists = true) {
+                                    c10::optional<Tensor> rowmap = c10::nullopt, bool with_row_lists = true,
+                                    int64_t out_rows = -1) {
     TORCH_CHECK(device.is_cuda(), "DeviceCsr lives on a GPU");
     TORCH_CHECK(rowptr.dim() == 1 && col.dim() == 1 && rowptr.numel() == rows + 1, "rowptr must have rows+1 entries");
     auto blk = std::make_shared<DeviceCsr>();
     blk->rows = rows;
+    blk->out_rows = out_rows < 0 ? rows : out_rows;
+    TORCH_CHECK(blk->out_rows >= rows && (blk->out_rows == rows || (rowmap.has_value() && rowmap->defined())),
+                "a block that stores fewer rows than its output has needs a rowmap");
     blk->cols = cols;
     blk->nnz = col.numel();
     blk->seg_nnz = (int32_t)seg_nnz;
@@ -212,9 +217,11 @@ Tensor block_spmm(DeviceCsr &A, const Tensor &mat, c10::optional<Tensor> optiona
         // caller must use the returned tensor
         out = optional_out->contiguous();
         require_gpu(out, "out");
-        TORCH_CHECK(out.dim() == 2 && out.size(0) == A.rows && out.size(1) == F && out.scalar_type() == mat.scalar_type(),
+        TORCH_CHECK(out.dim() == 2 && out.size(0) == A.out_rows && out.size(1) == F && out.scalar_type() == mat.scalar_type(),
                     "out must be [rows, F] of mat's dtype");
         accumulate = 1;
+    } else if (A.out_rows != A.rows) {
+        out = torch::zeros({A.out_rows, F}, mat.options());  // the rows that are not stored have no entries
     } else {
         out = torch::empty({A.rows, F}, mat.options());
     }
@@ -1039,12 +1046,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("version", []() { return std::string(cgnn_version()); });
     py::class_<DeviceCsr, std::shared_ptr<DeviceCsr>>(m, "DeviceCsr")
         .def(py::init([](Tensor rowptr, Tensor col, c10::optional<Tensor> value, int64_t rows, int64_t cols,
-                         torch::Device device, int64_t seg_nnz, c10::optional<Tensor> rowmap) {
-                 return make_csr(rowptr, col, value, rows, cols, device, seg_nnz, rowmap);
+                         torch::Device device, int64_t seg_nnz, c10::optional<Tensor> rowmap, int64_t out_rows) {
+                 return make_csr(rowptr, col, value, rows, cols, device, seg_nnz, rowmap, true, out_rows);
              }),
              py::arg("rowptr"), py::arg("col"), py::arg("value"), py::arg("rows"), py::arg("cols"),
-             py::arg("device"), py::arg("seg_nnz") = 0, py::arg("rowmap") = py::none())
+             py::arg("device"), py::arg("seg_nnz") = 0, py::arg("rowmap") = py::none(), py::arg("out_rows") = -1)
         .def_readonly("rowmap", &DeviceCsr::rowmap)
+        .def_readonly("out_rows", &DeviceCsr::out_rows)
         .def_readonly("rows", &DeviceCsr::rows)
         .def_readonly("cols", &DeviceCsr::cols)
         .def_readonly("nnz", &DeviceCsr::nnz)

@@ -123,6 +123,17 @@ class CompressGraph():
                 cp, row, val = g.csc()
                 return rt.DeviceCsr(cp, row, val, g.sparse_size(1), g.sparse_size(0), dev, seg)
 
+            def level(rp, ci, val, rows, cols):
+                """A rule level as the device reads it: only the rows that have entries (the rules
+                of that level; the reference pads every level to all R rule rows,
+                src/offline/csrc/partition.h:175-203), each with the rule row it updates."""
+                rp = rp.cpu()
+                lens = rp[1:] - rp[:-1]
+                live = torch.nonzero(lens).flatten()
+                packed = torch.zeros(live.numel() + 1, dtype=rp.dtype)
+                packed[1:] = torch.cumsum(lens[live], 0)
+                return rt.DeviceCsr(packed, ci, val, live.numel(), cols, dev, seg, live, rows)
+
             V, R = self.vertex_cnt, self.rule_cnt
             host = lambda triple: tuple(t.cpu().numpy() for t in triple)
             t = torch.from_numpy
@@ -137,8 +148,8 @@ class CompressGraph():
                 rules_bwd = rt.DeviceCsr(t(rp), t(ci), t(val), R, V, dev, seg)
                 plan = rt.PropagationPlan(V, R, rules_fwd, [], rules_bwd, [])
             else:
-                plan = rt.PropagationPlan(V, R, fwd(self.r2v_graph), [fwd(g) for g in self.r2r_graph],
-                                          bwd(self.v2r_graph), [bwd(g) for g in self.r2r_graph])
+                plan = rt.PropagationPlan(V, R, fwd(self.r2v_graph), [level(*g.csr(), R, R) for g in self.r2r_graph],
+                                          bwd(self.v2r_graph), [level(*g.csc(), R, R) for g in self.r2r_graph])
             if getattr(self, "keep_split_blocks", False):
                 # the vertex stages as two launches each (plan.fuse_final = False)
                 plan.set_split_blocks(fwd(self.v2v_graph), fwd(self.v2r_graph), bwd(self.v2v_graph), bwd(self.r2v_graph))

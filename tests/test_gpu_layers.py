@@ -246,6 +246,40 @@ def test_plan_feature_sweep(F, method, fold, fuse):
             other.edge_index.plan().fuse_final = False
 
 
+def test_rule_levels_are_stored_without_their_padding():
+    """One launch per level (the form kept for hierarchies too deep to fold): the reference pads
+    every level to all R rule rows (src/offline/csrc/partition.h:175-203); the device form of a level
+    holds only the rules of that level, each with the row it updates, and the chain over the
+    levels gives the oracle's bits in a forced row schedule, forward and gradient."""
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnData
+    v, e = off.gen_copy_model(3000, 9.8, 0.7, 2)
+    V = len(v) - 1
+    m = np.ones(V, bool)
+    rng = np.random.default_rng(8)
+    x_np = rng.standard_normal((V, 48)).astype(np.float32)
+    data = CompressgnnData(x_np, (v, e), np.zeros(V, np.int64), m, m, m, graph_type="csr", min_pair_frequency=3,
+                           threshold=0, max_depth=8, min_edge=0, verbose=False)
+    graph = data.edge_index
+    assert graph.step >= 2, "the fixture should have several rule levels"
+    fwd_blocks, bwd_blocks = _np_blocks(graph)
+    g_np = rng.standard_normal(x_np.shape).astype(np.float32)
+    want, want_g = oracle.compress_spmm_forward(fwd_blocks, x_np), oracle.compress_spmm_backward(bwd_blocks, g_np)
+    per_level = [int(np.count_nonzero(np.diff(b[0]))) for b in fwd_blocks["r2r"]]
+    data.to(DEV)
+    graph.fold_levels = False
+    plan = graph.plan()
+    assert not graph.levels_folded and len(plan.r2r) == graph.step == len(plan.r2r_t)
+    R = data.rule_cnt
+    assert [b.rows for b in plan.r2r] == per_level and all(b.out_rows == R and b.rows < R for b in plan.r2r + plan.r2r_t)
+    plan.method = "row_schedule"
+    out, gx = plan.forward(data.x), plan.backward(torch.from_numpy(g_np).to(DEV))
+    assert np.array_equal(out.cpu().numpy(), want) and np.array_equal(gx.cpu().numpy(), want_g)
+    plan.method = "nnz_schedule"
+    assert_within(plan.forward(data.x).cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+    assert_within(plan.backward(torch.from_numpy(g_np).to(DEV)).cpu().numpy(), want_g, rtol=1e-5, atol=1e-6)
+
+
 def test_propagation_replays_from_a_captured_graph():
     """Forward and gradient propagation make no host read, no memset and no allocation outside
     torch's allocator, so a step can be captured in a graph; every replay, with eager work and
