@@ -422,6 +422,7 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
     from CompressgnnCluster import Compressgnn_Cluster
     from CompressgnnData import CompressgnnData
     from CompressgnnReconstruct import Compressgnn_Reconstruct
+    from GatheredPropagate import GatheredPropagate
     from KPropagate import KPropagate
 
     dev = torch.device("cuda:0")
@@ -509,6 +510,46 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
             layers[1](h, epochs)
             c4_check_clusters(torch, layers, (p0, p1), checks)
         del p0, p1, h
+    # The same model with the first layer's reconstruct + ReLU and the second layer's propagation
+    # composed (GatheredPropagate: the propagation gathers from relu(H + b), a matrix of one row per
+    # cluster, through the index; the [N, hidden] rows are never written).  Same parameters from the
+    # same seed, same sums in the same order: the losses are those of the layer sequence above.
+    del layers, opt
+    torch.cuda.empty_cache()
+    torch.manual_seed(0)
+    layers = torch.nn.ModuleList([Layer(C4_F, C4_HIDDEN), Layer(C4_HIDDEN, C4_CLASSES)]).to(dev)
+    opt = torch.optim.Adam(layers.parameters(), lr=0.01)
+    gathered = GatheredPropagate()
+    torch.cuda.reset_peak_memory_stats()
+
+    def composed_epoch(k):
+        opt.zero_grad(set_to_none=True)
+        first, second = layers
+        p = first.P(x=x, edge_index=graph, edge_weight=None, vertex_cnt=data.vertex_cnt, rule_cnt=data.rule_cnt)
+        reps, index = first.cluster(p, epoch=k)
+        small = (Fn.linear(reps, first.lin.weight, None) + first.lin.bias).relu()
+        p = gathered(small, index, graph)
+        reps, index = second.cluster(p, epoch=k)
+        out = second.reconstruct(Fn.linear(reps, second.lin.weight, None), index, bias=second.lin.bias)
+        loss = -Fn.log_softmax(out, dim=1).gather(1, y.unsqueeze(1)).mean()
+        loss.backward()
+        opt.step()
+        return loss
+
+    c_losses, c_ms = [], []
+    for k in range(epochs + 1):
+        torch.cuda.synchronize()
+        t0 = time.time()
+        loss = composed_epoch(k)
+        torch.cuda.synchronize()
+        c_ms.append((time.time() - t0) * 1e3)
+        c_losses.append(float(loss.detach()))
+        log("[bench] C4 composed epoch %d: %.1f ms, loss %.4f" % (k, c_ms[-1], c_losses[-1]))
+    composed = dict(ms_per_epoch=float(np.mean(c_ms[1:])), epoch_ms=c_ms, loss=c_losses,
+                    peak_hbm_bytes=int(torch.cuda.max_memory_allocated()),
+                    max_loss_difference_to_the_layer_sequence=float(np.abs(np.array(c_losses) - np.array(losses)).max()))
+    if not composed["max_loss_difference_to_the_layer_sequence"] <= 1e-4:
+        raise RuntimeError("C4: the composed model's losses %s differ from the layer sequence's %s" % (c_losses, losses))
     return {
         "metric": "gcn_2layer_epoch_ms_C4", "value": float(np.mean(timed)), "unit": "ms", "n_gpus": 1,
         "steps": epochs, "warmup": 1, "ms_per_step": float(np.mean(timed)), "higher_is_better": False,
@@ -520,6 +561,7 @@ def bench_c4(torch, vertices, epochs, refresh_interval):
                    "rules": int(data.rule_cnt), "compressed_edges": int(data.edge_cnt), "levels": int(graph.step)},
         "detail": {"epoch_ms": ms, "loss": losses, "cluster_refreshes": refreshed,
                    "peak_hbm_bytes": peak, "checks": checks["checks"],
+                   "reconstruct_relu_propagate_composed": composed,
                    "active_clusters": [int(layers[0].cluster.active_bucket), int(layers[1].cluster.active_bucket)],
                    "host_seconds": times},
     }

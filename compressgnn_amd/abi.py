@@ -19,7 +19,7 @@ EXPORTS = [
     "cgnn_last_error", "cgnn_version",
     "cgnn_spmm_schedule", "cgnn_spmm_run_length", "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
     "cgnn_spmm_static_scratch_bytes", "cgnn_spmm_static_init", "cgnn_spmm_static",
-    "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows",
+    "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows", "cgnn_narrow_ids", "cgnn_csr_compose_columns",
     "cgnn_csr_transpose_workspace_bytes", "cgnn_csr_transpose_device",
     "cgnn_compress_batch_workspace_bytes", "cgnn_compress_csr_batch_device",
     "cgnn_lsh_scan_workspace_bytes", "cgnn_lsh_hash", "cgnn_lsh_scan", "cgnn_lsh_finish",

@@ -1181,6 +1181,41 @@ unsigned grid_for(int64_t n) {
     return (unsigned)(b > 16384 ? 16384 : b);
 }
 
+// narrow[c] = ids[c] as int32 (an id outside [0, groups) is replaced by the nearest valid one and
+// reported): the table the composition below gathers from, half the size of the int64 ids.
+__global__ void narrow_ids_kernel(const int64_t *__restrict__ ids, int64_t n, int64_t groups, int32_t *__restrict__ narrow,
+                                  int32_t *__restrict__ bad) {
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < n; c += (int64_t)gridDim.x * blockDim.x) {
+        int64_t id = ids[c];
+        if (id < 0 || id >= groups) {
+            if (bad) *bad = 1;  // every writer stores the same value
+            id = id < 0 ? 0 : groups - 1;
+        }
+        narrow[c] = (int32_t)id;
+    }
+}
+
+// out[e] = narrow[col[e]] for the columns below first_cols, the other columns unchanged.  Four
+// entries per thread, their table reads in flight together.
+__global__ void compose_columns_kernel(const int32_t *__restrict__ col, int64_t nnz, int64_t first_cols,
+                                       const int32_t *__restrict__ narrow, int32_t *__restrict__ out) {
+    const int64_t quads = nnz / 4;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
+        const int4 c = reinterpret_cast<const int4 *>(col)[q];
+        int4 r;
+        r.x = c.x < first_cols ? narrow[c.x] : c.x;
+        r.y = c.y < first_cols ? narrow[c.y] : c.y;
+        r.z = c.z < first_cols ? narrow[c.z] : c.z;
+        r.w = c.w < first_cols ? narrow[c.w] : c.w;
+        reinterpret_cast<int4 *>(out)[q] = r;
+    }
+    const int64_t e = quads * 4 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < nnz) {
+        const int32_t c = col[e];
+        out[e] = c < first_cols ? narrow[c] : c;
+    }
+}
+
 }  // namespace
 
 // Entry used by the cluster reductions (unit values; mask: 0 none, 1 the rows of M, where M <= 0 drops
@@ -1346,6 +1381,29 @@ extern "C" int cgnn_csr_prepare_i64(int64_t rows, int64_t nnz, const int64_t *ro
                            rowptr64, rows, nnz, rowidx);
     }
     return check_launch("csr_prepare");
+}
+
+extern "C" int cgnn_narrow_ids(int64_t n, const int64_t *ids, int64_t groups, int32_t *narrow, int32_t *bad_id,
+                               cgnn_stream_t stream) {
+    const int64_t lim = (int64_t)INT32_MAX - 65536;
+    CGNN_REQUIRE(n >= 0 && n < lim && groups >= 1 && groups < lim, "cgnn_narrow_ids: sizes must be in [0, 2^31 - 65536), at least one group");
+    if (n == 0) return CGNN_OK;
+    CGNN_REQUIRE(ids && narrow, "cgnn_narrow_ids: null array");
+    hipLaunchKernelGGL(narrow_ids_kernel, dim3(grid_for(n)), dim3(kBlock), 0, stream, ids, n, groups, narrow, bad_id);
+    return check_launch("narrow_ids");
+}
+
+extern "C" int cgnn_csr_compose_columns(int64_t nnz, const int32_t *colidx, int64_t first_cols, const int32_t *narrow_ids,
+                                        int32_t *out, cgnn_stream_t stream) {
+    const int64_t lim = (int64_t)INT32_MAX - 65536;
+    CGNN_REQUIRE(nnz >= 0 && nnz < lim && first_cols >= 0 && first_cols < lim, "cgnn_csr_compose_columns: sizes must be in [0, 2^31 - 65536)");
+    if (nnz == 0) return CGNN_OK;
+    CGNN_REQUIRE(colidx && narrow_ids && out, "cgnn_csr_compose_columns: null array");
+    CGNN_REQUIRE((reinterpret_cast<uintptr_t>(colidx) | reinterpret_cast<uintptr_t>(out)) % 16 == 0,
+                 "cgnn_csr_compose_columns: colidx and out must be 16-byte aligned");
+    hipLaunchKernelGGL(compose_columns_kernel, dim3(grid_for((nnz + 3) / 4)), dim3(kBlock), 0, stream, colidx, nnz, first_cols,
+                       narrow_ids, out);
+    return check_launch("csr_compose_columns");
 }
 
 extern "C" int cgnn_csr_expand_rows(int64_t rows, int64_t nnz, const int32_t *rowptr, int32_t *rowidx,

@@ -323,6 +323,16 @@ struct PropagationPlan {
     int kernel = CGNN_SPMM_AUTO;
     std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
     StageTimer timer;
+    // The forward blocks with their vertex columns sent through a cluster assignment
+    // (propagate_forward_gathered), kept for the index tensors they were made for: an
+    // assignment lasts until the next refresh, and a model may hold one per layer.
+    struct Composed {
+        c10::weak_intrusive_ptr<c10::TensorImpl> index;
+        uint32_t version;
+        int64_t groups;
+        std::shared_ptr<DeviceCsr> rules, stage;
+    };
+    std::deque<Composed> composed;
 
     void adopt(const std::shared_ptr<DeviceCsr> &block) {
         if (block) block->scratch = scratch;
@@ -379,6 +389,84 @@ Tensor propagate_forward(PropagationPlan &p, Tensor x) {
     for (size_t i = 0; i < p.r2r.size(); ++i)
         rule_out = timed_spmm(p, "fwd.level" + std::to_string(i), *p.r2r[i], rule_out, rule_out);
     return final_stage(p, "fwd.", p.vertex_stage.get(), p.v2r, rule_out, p.v2v, x);
+}
+
+// A copy of a block that shares everything but the column numbers: the columns below
+// `first_cols` go through `index` (cgnn_csr_compose_columns).
+std::shared_ptr<DeviceCsr> compose_block(const DeviceCsr &A, const Tensor &narrow, int64_t first_cols, int64_t cols) {
+    auto blk = std::make_shared<DeviceCsr>(A);
+    blk->cols = cols;
+    if (A.nnz > 0) {
+        blk->colidx = torch::empty_like(A.colidx);
+        ok(cgnn_csr_compose_columns(A.nnz, A.colidx.data_ptr<int32_t>(), first_cols, narrow.data_ptr<int32_t>(),
+                                    blk->colidx.data_ptr<int32_t>(), current_stream(narrow)),
+           "csr_compose_columns");
+    }
+    return blk;
+}
+
+// out = A * reps[index] over the compressed graph without reps[index]: the forward chain of
+// propagate_forward on blocks whose vertex columns name the representative of the vertex.
+// reps: [groups, F]; index: int64 [vertex_cnt] with values in [0, groups).  The same sums in the
+// same order as propagate_forward(reps.index_select(0, index)): the same bits.  The composed
+// blocks are made on the first call for an index tensor (one host read: the ids are checked)
+// and kept until that tensor is written to or freed.  Stage names: fwd.rules, fwd.level<i>, fwd.final.
+Tensor propagate_forward_gathered(PropagationPlan &p, Tensor reps, Tensor index) {
+    require_gpu(reps, "reps");
+    require_gpu(index, "index");
+    TORCH_CHECK(reps.dim() == 2 && reps.size(0) >= 1, "reps must be [groups, F] with at least one group");
+    TORCH_CHECK(index.dim() == 1 && index.numel() == p.V && index.scalar_type() == torch::kInt64 && index.is_contiguous() &&
+                    index.device() == reps.device(),
+                "index must be a contiguous int64 tensor [vertex_cnt] on the device of reps");
+    TORCH_CHECK(p.fused(), "propagation from representatives needs the fused vertex stage (plan.fuse_final = True)");
+    reps = reps.contiguous();
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(reps.device());
+    const int64_t groups = reps.size(0), F = reps.size(1);
+    std::shared_ptr<DeviceCsr> rules, stage;
+    for (auto it = p.composed.begin(); it != p.composed.end();) {
+        if (it->index.expired()) {
+            it = p.composed.erase(it);
+            continue;
+        }
+        if (it->index._unsafe_get_target() == index.unsafeGetTensorImpl() && it->version == index._version() &&
+            it->groups == groups) {
+            rules = it->rules;
+            stage = it->stage;
+            break;
+        }
+        ++it;
+    }
+    if (!stage) {
+        Tensor bad = torch::zeros({1}, index.options().dtype(torch::kInt32));
+        Tensor narrow = torch::empty({p.V}, index.options().dtype(torch::kInt32));
+        ok(cgnn_narrow_ids(p.V, index.data_ptr<int64_t>(), groups, narrow.data_ptr<int32_t>(), bad.data_ptr<int32_t>(),
+                           current_stream(index)),
+           "narrow_ids");
+        rules = compose_block(*p.r2v, narrow, p.V, groups);
+        stage = compose_block(*p.vertex_stage, narrow, p.V, p.vertex_stage->cols);
+        TORCH_CHECK(bad.item<int32_t>() == 0, "propagation from representatives: the index holds a cluster id outside [0, ", groups, ")");
+        if (!index.is_inference()) {
+            p.composed.push_front(PropagationPlan::Composed{c10::weak_intrusive_ptr<c10::TensorImpl>(index.getIntrusivePtr()),
+                                                           index._version(), groups, rules, stage});
+            while (p.composed.size() > 4) p.composed.pop_back();
+        }
+    }
+    Tensor rule_out = timed_spmm(p, "fwd.rules", *rules, reps, c10::nullopt);
+    for (size_t i = 0; i < p.r2r.size(); ++i)
+        rule_out = timed_spmm(p, "fwd.level" + std::to_string(i), *p.r2r[i], rule_out, rule_out);
+    Tensor out = torch::empty({p.V, F}, reps.options());
+    if (out.numel() == 0) return out;
+    const int dtype = dtype_code(reps);
+    size_t bytes = 0;
+    Tensor ws = stage->workspace(F, dtype, p.kernel, &bytes);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(current_stream(reps));
+    const int id = p.timer.open("fwd.final", stream);
+    cgnn_csr a = stage->view();
+    ok(cgnn_spmm_dual(&a, p.V, dtype, reps.data_ptr(), rule_out.data_ptr(), out.data_ptr(), F, p.kernel, ws.data_ptr(), bytes,
+                      current_stream(reps)),
+       "spmm_dual");
+    p.timer.close(id, stream);
+    return out;
 }
 
 // layer/CompressgnnSPMM.py:65-86 (the working branch, lines 80-85).  Stage names as in
@@ -1135,5 +1223,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def_readonly("r2v_t", &PropagationPlan::r2v_t)
         .def_readonly("r2r_t", &PropagationPlan::r2r_t)
         .def("forward", &propagate_forward)
+        .def("forward_gathered", &propagate_forward_gathered, py::arg("reps"), py::arg("index"),
+             "out = A * reps[index] without the [vertex_cnt, F] matrix reps[index]")
         .def("backward", &propagate_backward);
 }

@@ -148,6 +148,22 @@ int cgnn_csr_prepare_i64(int64_t rows, int64_t nnz, const int64_t *rowptr64,
                          const int64_t *col64, int32_t *rowptr32, int32_t *col32,
                          int32_t *rowidx, cgnn_stream_t stream);
 
+/* Column numbers of a block composed with a cluster assignment: out[e] = narrow_ids[colidx[e]]
+ * where colidx[e] < first_cols, colidx[e] otherwise.  With these columns a product gathers row
+ * ids[c] of a matrix of representatives where the block's own columns would gather row c of the
+ * N x F matrix reps[ids] -- the rows Compressgnn_Reconstruct writes
+ * (layer/CompressgnnReconstruct.py:34-42) and the next propagation reads
+ * (layer/CompressgnnPropagation.py:62-67) -- so that matrix need not exist.  No counterpart in the
+ * reference, whose layers hand each other dense tensors.  narrow_ids (first_cols entries, every
+ * one in [0, groups) of the matrix of representatives) comes from cgnn_narrow_ids, which turns
+ * the int64 ids of an assignment into int32, replaces an id outside [0, groups) by the nearest
+ * valid one and stores 1 to *bad_id (may be NULL) when it meets one.  colidx and out: 16-byte
+ * aligned. */
+int cgnn_narrow_ids(int64_t n, const int64_t *ids, int64_t groups, int32_t *narrow_ids, int32_t *bad_id,
+                    cgnn_stream_t stream);
+int cgnn_csr_compose_columns(int64_t nnz, const int32_t *colidx, int64_t first_cols, const int32_t *narrow_ids,
+                             int32_t *out, cgnn_stream_t stream);
+
 /* rowidx[e] = row of non-zero e, from an int32 rowptr. */
 int cgnn_csr_expand_rows(int64_t rows, int64_t nnz, const int32_t *rowptr,
                          int32_t *rowidx, cgnn_stream_t stream);

@@ -611,3 +611,50 @@ def test_reference_method_strings_are_hints():
     # a forced row schedule stays available under this build's own name, bit-exact with the oracle
     forced = rt.DeviceCsr(tv, te, tw, rows, cols, torch.device(DEV)).spmm(tx, None, "row_schedule")
     assert np.array_equal(forced.cpu().numpy(), want)
+
+
+def test_propagation_from_representatives_equals_propagation_of_the_written_rows():
+    """GatheredPropagate(small, index, graph) against KPropagate on small[index]: the same bits,
+    forward and gradient, for an assignment of Compressgnn_Cluster and for an index from
+    elsewhere, folded and launch-per-level plans; an id that names no cluster is refused; a new
+    assignment is noticed."""
+    from CompressgnnCluster import Compressgnn_Cluster
+    from GatheredPropagate import GatheredPropagate
+    from KPropagate import KPropagate
+    for fold in (True, False):
+        data, _ = _make_data("copy", 64, True, 3, seed=6)
+        data.to(DEV)
+        graph = data.edge_index
+        graph.fold_levels = fold
+        V, F = data.vertex_cnt, 64
+        torch.manual_seed(3)
+        cluster = Compressgnn_Cluster(in_feature=F, param_H=7, training=True, cache=False).to(DEV)
+        reps, index = cluster(data.x)
+        C = reps.size(0)
+        g = torch.randn(V, F, device=DEV)
+        for idx in (index, torch.randint(0, C, (V,), device=DEV)):
+            small = torch.randn(C, F, device=DEV, requires_grad=True)
+            out = GatheredPropagate()(small.relu(), idx, graph)
+            (d_small,) = torch.autograd.grad(out, small, g)
+            small2 = small.detach().clone().requires_grad_()
+            rows = small2.relu().index_select(0, idx)
+            want = KPropagate()(rows, graph, None, data.vertex_cnt, data.rule_cnt)
+            (d_want,) = torch.autograd.grad(want, small2, g)
+            assert torch.equal(out, want)
+            # the dense path sums a cluster's gradient through index_select's backward (atomics in
+            # torch); the member-list sum has a fixed order
+            ref = torch.zeros(C, F, dtype=torch.float64, device=DEV).index_add_(
+                0, idx, graph.plan().backward(g).double()) * (small.detach() > 0)
+            assert_within(d_small.cpu().numpy(), ref.cpu().numpy(), rtol=1e-5, atol=1e-6)
+            assert_within(d_want.cpu().numpy(), ref.cpu().numpy(), rtol=1e-4, atol=1e-5)
+        # a refreshed assignment (another tensor) is composed anew
+        reps_b, index_b = cluster(data.x * 1.5 + 0.1)
+        small = torch.randn(reps_b.size(0), F, device=DEV)
+        assert torch.equal(GatheredPropagate()(small, index_b, graph),
+                           KPropagate()(small.index_select(0, index_b), graph, None, data.vertex_cnt, data.rule_cnt))
+        bad = index_b.clone()
+        bad[5] = reps_b.size(0) + 3
+        with pytest.raises(RuntimeError, match="outside"):
+            GatheredPropagate()(small, bad, graph)
+        with pytest.raises(ValueError):
+            GatheredPropagate()(small, index_b[:-1], graph)
