@@ -658,3 +658,11 @@ def test_propagation_from_representatives_equals_propagation_of_the_written_rows
             GatheredPropagate()(small, bad, graph)
         with pytest.raises(ValueError):
             GatheredPropagate()(small, index_b[:-1], graph)
+    # a graph without rules: the rule stage has nothing to do
+    data, _ = _make_data("chung_lu", 32, True, 10 ** 6, seed=2)
+    assert data.rule_cnt == 0
+    data.to(DEV)
+    idx = torch.randint(0, 50, (data.vertex_cnt,), device=DEV)
+    small = torch.randn(50, 32, device=DEV)
+    assert torch.equal(GatheredPropagate()(small, idx, data.edge_index),
+                       KPropagate()(small.index_select(0, idx), data.edge_index, None, data.vertex_cnt, data.rule_cnt))
