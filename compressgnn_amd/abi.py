@@ -17,7 +17,7 @@ SPMM_AUTO, SPMM_ROW, SPMM_NNZ = 0, 1, 2
 
 EXPORTS = [
     "cgnn_last_error", "cgnn_version",
-    "cgnn_spmm_schedule", "cgnn_spmm_run_length", "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
+    "cgnn_spmm_schedule", "cgnn_spmm_run_length", "cgnn_spmm_run_starts", "cgnn_spmm_workspace_bytes", "cgnn_spmm", "cgnn_spmm_dual",
     "cgnn_spmm_static_scratch_bytes", "cgnn_spmm_static_init", "cgnn_spmm_static",
     "cgnn_csr_prepare_i64", "cgnn_csr_expand_rows", "cgnn_narrow_ids", "cgnn_csr_compose_columns",
     "cgnn_csr_transpose_workspace_bytes", "cgnn_csr_transpose_device",
@@ -41,6 +41,7 @@ class CsrStruct(ctypes.Structure):
         ("rowmap", ctypes.c_void_p),
         ("cut_rows", ctypes.c_void_p), ("empty_rows", ctypes.c_void_p),
         ("n_cut_rows", ctypes.c_int32), ("n_empty_rows", ctypes.c_int32),
+        ("run_start", ctypes.c_void_p),
     ]
 
 
@@ -103,6 +104,7 @@ class DeviceCsr:
         self.rowmap = rowmap  # int32 [rows] on the device: stored row g is row rowmap[g] of the output
         self.nnz = int(colidx.numel())
         self.max_row_nnz, self.seg_nnz = int(max_row_nnz), int(seg_nnz)
+        self.run_start = None  # int32 on the device, see make_run_starts
         self._ws = {}
 
     @classmethod
@@ -130,7 +132,19 @@ class DeviceCsr:
         s.val = self.val.data_ptr() if (self.val is not None and self.nnz) else 0
         s.max_row_nnz, s.seg_nnz = self.max_row_nnz, self.seg_nnz
         s.rowmap = self.rowmap.data_ptr() if self.rowmap is not None else 0
+        s.run_start = self.run_start.data_ptr() if self.run_start is not None else 0
         return s
+
+    def make_run_starts(self):
+        """Builds the optional table of run starts through cgnn_spmm_run_starts (the block needs
+        rowidx); the products that follow read it."""
+        self.run_start = None
+        s = self.struct()
+        runs = lib().cgnn_spmm_run_length(ctypes.byref(s))
+        table = torch.empty((self.nnz + runs - 1) // runs + 1, dtype=torch.int32, device=self.rowptr.device)
+        check(lib().cgnn_spmm_run_starts(ctypes.byref(s), ptr(table), stream_of(table)))
+        self.run_start = table
+        return table
 
     def workspace(self, F, dtype, kernel):
         """Scratch for one (F, dtype, kernel), cached on the block (per stream use is the

@@ -93,6 +93,7 @@ struct SpmmArgs {
     const int32_t *cut_rows;    // spmm_fixup_rows_kernel: the stored rows that the runs cut, ascending
     const int32_t *empty_rows;  // and the stored rows without entries
     int32_t n_cut_rows, n_empty_rows;
+    const int32_t *run_start;   // nnz schedule: first non-zero of every run, [nseg + 1], or NULL (run_boundary)
 };
 
 // carry_row values below zero: the run carries nothing, or its carry was added to that
@@ -430,8 +431,13 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     if constexpr (LPR == kWave) seg = __builtin_amdgcn_readfirstlane(seg);
     int e0 = 0, e1 = 0;
     if (seg < a.nseg) {
-        e0 = run_boundary(a, seg * a.seg_nnz);
-        e1 = run_boundary(a, (seg + 1) * a.seg_nnz);
+        if (a.run_start != nullptr) {  // one load instead of two dependent ones
+            e0 = a.run_start[seg];
+            e1 = a.run_start[seg + 1];
+        } else {
+            e0 = run_boundary(a, seg * a.seg_nnz);
+            e1 = run_boundary(a, (seg + 1) * a.seg_nnz);
+        }
     }
     // e0 >= e1 inside the list cannot happen for a well-formed CSR
     const bool active = e0 < e1;
@@ -443,6 +449,8 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     bool continues = false;
     if (active) {
         cur = a.rowidx[e0];
+        // asked for now, beside the entries, and looked at when the run is done
+        const int row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
         if constexpr (LPR >= kUnroll && sizeof(T) == 4) {
             // As in the row schedule: the lanes of the group load one entry each, and the
             // entries reach all lanes through the LDS crossbar.
@@ -538,7 +546,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                 }
             }
         }
-        continues = (e1 < a.nnz) && (a.rowidx[e1] == cur);
+        continues = row_behind == cur;
         if (!continues) write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
     }
     // The carries of one row are added per workgroup: the first of its lane groups that
@@ -1115,6 +1123,7 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     auto level_carries = [&](int k) { return reinterpret_cast<T *>(base + levels.carry_off[k]); };
     a.nseg = (int32_t)nseg;
     a.seg_nnz = seg;
+    a.run_start = A->run_start;
     a.carry_row = nseg > 0 ? level_rows(0) : nullptr;
     a.carry = nseg > 0 ? level_carries(0) : nullptr;
     a.merge_stride = runs_per_workgroup;
@@ -1158,6 +1167,21 @@ __global__ void narrow_i64_kernel(const int64_t *__restrict__ src, int32_t *__re
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
          i += (int64_t)gridDim.x * blockDim.x)
         dst[i] = (int32_t)src[i];
+}
+
+// run_start[s] = where the run of the nnz schedule that covers position s * seg begins.
+__global__ void run_starts_kernel(const int32_t *__restrict__ rowptr, const int32_t *__restrict__ rowidx, int32_t nnz,
+                                  int32_t seg, int64_t n, int32_t *__restrict__ run_start) {
+    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (s >= n) return;
+    const int64_t e = s * seg;
+    if (e >= nnz) {
+        run_start[s] = nnz;
+        return;
+    }
+    const int r = rowidx[e];
+    const int s0 = rowptr[r];
+    run_start[s] = (rowptr[r + 1] - s0 <= seg) ? s0 : (int32_t)e;
 }
 
 // rowidx[e] = largest r with rowptr[r] <= e (rows without entries are skipped).
@@ -1404,6 +1428,18 @@ extern "C" int cgnn_csr_compose_columns(int64_t nnz, const int32_t *colidx, int6
     hipLaunchKernelGGL(compose_columns_kernel, dim3(grid_for((nnz + 3) / 4)), dim3(kBlock), 0, stream, colidx, nnz, first_cols,
                        narrow_ids, out);
     return check_launch("csr_compose_columns");
+}
+
+extern "C" int cgnn_spmm_run_starts(const cgnn_csr *A, int32_t *run_start, cgnn_stream_t stream) {
+    int rc = check_csr(A, "cgnn_spmm_run_starts");
+    if (rc != CGNN_OK) return rc;
+    CGNN_REQUIRE(run_start != nullptr, "cgnn_spmm_run_starts: null array");
+    CGNN_REQUIRE(A->nnz == 0 || A->rowidx != nullptr, "cgnn_spmm_run_starts: the block needs rowidx");
+    const int seg = seg_len(A);
+    const int64_t n = ceil_div(A->nnz, seg) + 1;
+    hipLaunchKernelGGL(run_starts_kernel, dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, stream, A->rowptr,
+                       A->rowidx, (int32_t)A->nnz, seg, n, run_start);
+    return check_launch("spmm_run_starts");
 }
 
 extern "C" int cgnn_csr_expand_rows(int64_t rows, int64_t nnz, const int32_t *rowptr, int32_t *rowidx,

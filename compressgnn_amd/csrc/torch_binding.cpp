@@ -69,6 +69,7 @@ struct DeviceCsr {
     int32_t max_row_nnz = 0;
     int32_t seg_nnz = 0;
     Tensor cut_rows, empty_rows;  // the rows the runs of the nnz schedule cut / the rows without entries
+    Tensor run_start;  // nnz schedule: where every run begins (made with rowidx)
     std::shared_ptr<Scratch> scratch = std::make_shared<Scratch>();
 
     cgnn_csr view() const {
@@ -83,6 +84,7 @@ struct DeviceCsr {
         a.max_row_nnz = max_row_nnz;
         a.seg_nnz = seg_nnz;
         a.rowmap = rowmap.defined() ? rowmap.data_ptr<int32_t>() : nullptr;
+        a.run_start = run_start.defined() ? run_start.data_ptr<int32_t>() : nullptr;
         if (cut_rows.defined()) {
             a.cut_rows = cut_rows.data_ptr<int32_t>();  // a tensor without entries gives a pointer that is never read
             a.n_cut_rows = (int32_t)cut_rows.numel();
@@ -113,14 +115,22 @@ struct DeviceCsr {
 
     // rowidx (the row of every non-zero, as large as colidx) is read by the nnz schedule only:
     // it is made when a product first resolves to that schedule, on the product's stream.
+    // So is the table of run starts, which belongs to a run length as the row lists do.
     void ensure_rowidx(int kernel) {
-        if (nnz == 0 || rowidx.defined()) return;
+        if (nnz == 0 || (rowidx.defined() && run_start.defined())) return;
         if (cgnn_spmm_schedule(rows, nnz, max_row_nnz, kernel) != CGNN_SPMM_NNZ) return;
-        rowidx = torch::empty({nnz}, rowptr.options());
-        ok(cgnn_csr_expand_rows(rows, nnz, rowptr.data_ptr<int32_t>(), rowidx.data_ptr<int32_t>(),
-                                reinterpret_cast<cgnn_stream_t>(
-                                    c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(rowptr.device().index()).stream())),
-           "csr_expand_rows");
+        auto stream = reinterpret_cast<cgnn_stream_t>(
+            c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(rowptr.device().index()).stream());
+        if (!rowidx.defined()) {
+            rowidx = torch::empty({nnz}, rowptr.options());
+            ok(cgnn_csr_expand_rows(rows, nnz, rowptr.data_ptr<int32_t>(), rowidx.data_ptr<int32_t>(), stream),
+               "csr_expand_rows");
+        }
+        cgnn_csr a = view();
+        const int64_t K = cgnn_spmm_run_length(&a);
+        Tensor starts = torch::empty({(nnz + K - 1) / K + 1}, rowptr.options());
+        ok(cgnn_spmm_run_starts(&a, starts.data_ptr<int32_t>(), stream), "spmm_run_starts");
+        run_start = starts;
     }
 
     Tensor workspace(int64_t F, int dtype, int kernel, size_t *bytes) {
@@ -1148,9 +1158,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def_property("seg_nnz", [](DeviceCsr &self) { return self.seg_nnz; },
                       [](DeviceCsr &self, int32_t seg) {
                           self.seg_nnz = seg;
+                          self.run_start = Tensor();  // made again by the next product
                           if (self.cut_rows.defined()) self.list_rows();  // the lists belong to a run length
                       })
         .def_readonly("cut_rows", &DeviceCsr::cut_rows)
+        .def_readonly("run_start", &DeviceCsr::run_start)
         .def_readonly("empty_rows", &DeviceCsr::empty_rows)
         .def_readonly("rowptr", &DeviceCsr::rowptr)
         .def_readonly("colidx", &DeviceCsr::colidx)

@@ -76,6 +76,13 @@ typedef struct cgnn_csr {
     const int32_t *cut_rows;   /* [n_cut_rows] */
     const int32_t *empty_rows; /* [n_empty_rows] */
     int32_t n_cut_rows, n_empty_rows;
+    /* NNZ schedule, optional (NULL = every lane group finds its run from rowidx and rowptr, two
+     * dependent loads before it can read its first entry): the first non-zero of every run,
+     * [ceil(nnz / K) + 1] with K = cgnn_spmm_run_length(A).  run_start[s] for the position
+     * e = s * K is nnz if e >= nnz, else rowptr[r] if row r = rowidx[e] has at most K entries (a short
+     * row is never cut: the run begins with it), else e.  Must be exact when given (not checked).
+     * Results are unchanged. */
+    const int32_t *run_start;
 } cgnn_csr;
 
 const char *cgnn_last_error(void);
@@ -91,6 +98,10 @@ int cgnn_spmm_schedule(int64_t rows, int64_t nnz, int32_t max_row_nnz, int kerne
 /* Non-zeros per run of the NNZ schedule for this block (seg_nnz, or the default, rounded up to
  * what the kernels take). */
 int cgnn_spmm_run_length(const cgnn_csr *A);
+
+/* Fills run_start[ceil(nnz / K) + 1] (K = cgnn_spmm_run_length(A)) for a block that has rowidx: the
+ * optional table of cgnn_csr.run_start, as defined there.  No counterpart in the reference. */
+int cgnn_spmm_run_starts(const cgnn_csr *A, int32_t *run_start, cgnn_stream_t stream);
 
 /* Bytes of scratch cgnn_spmm needs for this block, feature width and schedule
  * (the carry-out rows of the NNZ schedule).  0 for the ROW schedule. */

@@ -350,3 +350,53 @@ def test_fixup_over_row_lists_reads_only_fresh_carries(seg):
     # the same block without the lists (the C ABI without cut_rows) gives the same bits
     plain = abi.DeviceCsr.from_host(rows, cols, vlist, elist, value, DEV, seg_nnz=seg)
     assert torch.equal(abi.spmm(plain, X, None, False, abi.SPMM_NNZ), got)
+
+
+@pytest.mark.parametrize("seg", [8, 32, 64])
+@pytest.mark.parametrize("F", [16, 128])
+def test_table_of_run_starts(seg, F):
+    """The optional table that tells every lane group of the nnz schedule where its run begins:
+    its entries against the definition worked out with numpy (the run that covers position s*K
+    begins with the row found there when that row has at most K entries, at s*K otherwise, and at
+    nnz behind the last entry), and the products with the table against those without: same bits,
+    plain and two-source, fresh and accumulating."""
+    import compressgnn_runtime as rt
+    rng = np.random.default_rng(100 + seg + F)
+    rows, cols = 2500, 700
+    vlist, elist, value = random_csr(rng, rows, cols, 7.0, skew=True)
+    row_len = np.repeat(np.diff(vlist), np.diff(vlist))
+    value = (value * 0.3 / np.sqrt(np.maximum(row_len, 1))).astype(np.float32)
+    nnz = len(elist)
+    x = rng.standard_normal((cols, F)).astype(np.float32)
+    X = torch.from_numpy(x).to(DEV)
+    A = abi.DeviceCsr.from_host(rows, cols, vlist, elist, value, DEV, seg_nnz=seg)
+    K = abi.lib().cgnn_spmm_run_length(__import__("ctypes").byref(A.struct()))
+    assert K == (seg + 3) // 4 * 4
+    without = abi.spmm(A, X, None, False, abi.SPMM_NNZ)
+    out0 = torch.from_numpy(rng.standard_normal((rows, F)).astype(np.float32)).to(DEV)
+    without_acc = abi.spmm(A, X, out0.clone(), True, abi.SPMM_NNZ)
+    split = cols // 2
+    X1 = torch.from_numpy(rng.standard_normal((cols - split, F)).astype(np.float32)).to(DEV)
+    without_dual = abi.spmm_dual(A, split, X[:split].contiguous(), X1, None, abi.SPMM_NNZ)
+    table = A.make_run_starts().cpu().numpy()
+    pos = np.arange((nnz + K - 1) // K + 1, dtype=np.int64) * K
+    inside = pos < nnz
+    row_of = np.searchsorted(vlist, pos[inside], side="right") - 1
+    start, length = vlist[row_of], vlist[row_of + 1] - vlist[row_of]
+    want = np.full(len(pos), nnz, dtype=np.int64)
+    want[inside] = np.where(length <= K, start, pos[inside])
+    assert np.array_equal(table, want.astype(np.int32))
+    assert (want[inside] < pos[inside]).any() and (want[inside] == pos[inside]).any()
+    assert torch.equal(abi.spmm(A, X, None, False, abi.SPMM_NNZ), without)
+    assert torch.equal(abi.spmm(A, X, out0.clone(), True, abi.SPMM_NNZ), without_acc)
+    assert torch.equal(abi.spmm_dual(A, split, X[:split].contiguous(), X1, None, abi.SPMM_NNZ), without_dual)
+    assert_within(without.cpu().numpy(), oracle.spmm(vlist, elist, value, x))
+    # a block of the operator module makes the same table with its first product in this schedule
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    B = rt.DeviceCsr(t(vlist), t(elist), t(value), rows, cols, torch.device(DEV), seg)
+    assert torch.equal(B.spmm(X, None, "nnz_schedule"), without)
+    assert np.array_equal(B.run_start.cpu().numpy(), table)
+    B.seg_nnz = 2 * seg  # another run length: another table, the same sums for the rows that stay whole
+    again = B.spmm(X, None, "nnz_schedule")
+    assert B.run_start.numel() == (nnz + 2 * K - 1) // (2 * K) + 1
+    assert_within(again.cpu().numpy(), oracle.spmm(vlist, elist, value, x))
