@@ -6,6 +6,7 @@ loader/compress_graph.py:6-57; on a GPU it additionally carries the propagation 
 from concurrent.futures import ThreadPoolExecutor
 
 import _paths  # noqa: F401
+import numpy as np
 import torch
 
 from compressgnn_offline import (csr_fold_levels, csr_fold_levels_bound, csr_hstack, csr_locality_order, csr_permute_rows, gen_degree,
@@ -41,6 +42,7 @@ class CompressGraph():
         self.keep_split_blocks = False   # plan(): also build the four vertex-stage blocks on their own
         self.keep_device_blocks = False  # plan(): leave the int64 blocks on the device
         self._plan = None
+        self._stage_orders = None        # the locality orders of the two vertex stages, once a plan has found them
 
     def __repr__(self):
         return 'CompressGraph'
@@ -158,9 +160,16 @@ class CompressGraph():
             # rows of the input follow each other and are processed on one XCD), which cuts
             # the misses in the per-XCD L2 caches; results do not depend on the order in the
             # row schedule, and in the nnz schedule only where a long row is cut into runs.
-            def ordered(first, second):
+            # The search for an order is the expensive part of a plan (most of 22 s at 18.5 M vertices)
+            # and depends on the blocks alone, so the graph keeps the two orders: a later plan() -- after
+            # another to(device), or after the dataset was saved and loaded -- only applies them.
+            kept = getattr(self, "_stage_orders", None) or {}
+
+            def ordered(which, first, second):
                 rp, ci, val = csr_hstack(first, second, V)
-                order = csr_locality_order(rp, ci)
+                order = kept.get(which)
+                if order is None or len(order) != len(rp) - 1:
+                    order = np.ascontiguousarray(csr_locality_order(rp, ci), dtype=np.int32)
                 return csr_permute_rows(rp, ci, val, order) + (order,)
 
             def stage(rp, ci, val, order):
@@ -177,8 +186,10 @@ class CompressGraph():
                 for block in self.blocks():
                     block.offload()
             with ThreadPoolExecutor(max_workers=2) as pool:
-                forward_job = pool.submit(ordered, *forward_blocks)
-                backward_job = pool.submit(ordered, *backward_blocks)
-                plan.set_vertex_stages(stage(*forward_job.result()), stage(*backward_job.result()))
+                forward_job = pool.submit(ordered, "forward", *forward_blocks)
+                backward_job = pool.submit(ordered, "backward", *backward_blocks)
+                forward_stage, backward_stage = forward_job.result(), backward_job.result()
+                self._stage_orders = {"forward": forward_stage[3], "backward": backward_stage[3]}
+                plan.set_vertex_stages(stage(*forward_stage), stage(*backward_stage))
             self._plan = plan
         return self._plan

@@ -666,3 +666,38 @@ def test_propagation_from_representatives_equals_propagation_of_the_written_rows
     small = torch.randn(50, 32, device=DEV)
     assert torch.equal(GatheredPropagate()(small, idx, data.edge_index),
                        KPropagate()(small.index_select(0, idx), data.edge_index, None, data.vertex_cnt, data.rule_cnt))
+
+
+def test_a_later_plan_applies_the_orders_the_first_one_found(tmp_path, monkeypatch):
+    """The locality orders of the two vertex stages depend on the blocks alone: the graph keeps them,
+    a dataset saved with torch.save carries them, and a plan built later (after loading, after
+    another to(device)) does not search again -- the search routine is made to raise here -- and
+    propagates to the same bits, forward and backward."""
+    import compress_graph
+    data, _ = _make_data("copy", 48, True, 3, seed=6)
+    assert data.edge_index._stage_orders is None
+    data.to(DEV)
+    graph = data.edge_index
+    plan = graph.plan()
+    V = data.vertex_cnt
+    for order in graph._stage_orders.values():
+        assert order.dtype == np.int32 and np.array_equal(np.sort(order), np.arange(V))
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    x = torch.randn(V, 48, device=DEV, generator=gen)
+    g = torch.randn(V, 48, device=DEV, generator=gen)
+    out, gx = plan.forward(x), plan.backward(g)
+    path = str(tmp_path / "prepared.pt")
+    torch.save(data, path)  # this test's own file
+    loaded = torch.load(path, weights_only=False)
+
+    def no_search(*_):
+        raise AssertionError("the locality order was searched for again")
+
+    monkeypatch.setattr(compress_graph, "csr_locality_order", no_search)
+    loaded.to(DEV)
+    again = loaded.edge_index.plan()
+    assert torch.equal(again.forward(x), out) and torch.equal(again.backward(g), gx)
+    graph.to(DEV)  # drops the plan, keeps the orders
+    assert graph._plan is None
+    once_more = graph.plan()
+    assert torch.equal(once_more.forward(x), out) and torch.equal(once_more.backward(g), gx)
