@@ -10,9 +10,12 @@ Pipeline (the reference's order): self loops -> normalised degrees of the uncomp
 graph -> batch compression -> saving filter -> depth filter -> weights of the compressed
 edges -> partition ("csr") or phase masks ("coo").
 """
+import copy
+
 import _paths  # noqa: F401
 import numpy as np
 import torch
+import torch.utils.data
 
 import compressgnn_offline as offline
 from compress_graph import CompressGraph
@@ -156,3 +159,30 @@ class CompressgnnData():
             self.edge_index = [e.to(device) for e in self.edge_index]
             self.edge_weight = [w.to(device) for w in self.edge_weight]
         return self
+
+
+class CompressgnnBatchData():
+    """A sequence of prepared datasets stored in one file (loader/CompressgnnData.py:203-209 of
+    the reference): `torch.save([data_0, data_1, ...], path)` of CompressgnnData objects made by
+    this library.  The file holds pickled objects, so it is opened with the unpickler: load only
+    files that this library wrote."""
+
+    def __init__(self, path):
+        self.data = torch.load(path, weights_only=False)
+        self.len = len(self.data)
+
+    def __len__(self):
+        return self.len
+
+
+class CompressgnnDataLoader(torch.utils.data.DataLoader):
+    """Hands out the datasets of a CompressgnnBatchData one per step
+    (loader/CompressgnnData.py:212-222): the loader walks the positions, and a step is a shallow
+    copy of the dataset at the first position of its batch, as in the reference."""
+
+    def __init__(self, data, **kwargs):
+        self.data = data
+        super().__init__(range(len(data)), collate_fn=self.__collate__, **kwargs)
+
+    def __collate__(self, batch):
+        return copy.copy(self.data.data[int(batch[0])])

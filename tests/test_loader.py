@@ -181,6 +181,31 @@ def test_a_prepared_dataset_survives_torch_save(tmp_path):
     assert torch.equal(again.edge_index.vertex_degree, data.edge_index.vertex_degree)
 
 
+def test_batch_data_and_its_loader(tmp_path):
+    """CompressgnnBatchData / CompressgnnDataLoader (loader/CompressgnnData.py:203-222 of the
+    reference): a list of prepared datasets in one file, handed out one per step as shallow
+    copies, in order or shuffled by the DataLoader's own arguments."""
+    import compressgnn_offline as off
+    from CompressgnnData import CompressgnnBatchData, CompressgnnDataLoader
+    parts = []
+    for seed, n in ((1, 300), (2, 500), (3, 400)):
+        v, e = off.gen_copy_model(n, 6.0, 0.7, seed)
+        mask = np.ones(n, dtype=bool)
+        parts.append(CompressgnnData(np.full((n, 2), float(seed), np.float32), (v, e), np.zeros(n, np.int64), mask, mask,
+                                     mask, graph_type="csr", min_pair_frequency=3, compression_backend="cpu"))
+    path = str(tmp_path / "batches.pt")
+    torch.save(parts, path)  # this test's own file
+    batches = CompressgnnBatchData(path)
+    assert len(batches) == 3
+    seen = list(CompressgnnDataLoader(batches))
+    assert [d.vertex_cnt for d in seen] == [300, 500, 400]
+    for got, want in zip(seen, batches.data):
+        assert got is not want and got.x is want.x and repr(got) == repr(want)  # a shallow copy
+        assert float(got.x[0, 0]) == float(want.x[0, 0])
+    shuffled = list(CompressgnnDataLoader(batches, shuffle=True, generator=torch.Generator().manual_seed(0)))
+    assert sorted(d.vertex_cnt for d in shuffled) == [300, 400, 500]
+
+
 def _binary_hierarchy(depth, width=2):
     """A compressed graph whose rules form `depth` levels of `width` rules each; every rule
     above the lowest level has all rules of the level below as children, so the vertices a
