@@ -53,6 +53,20 @@ class Propagate(torch.nn.Module):
         plan = self._coo_plans.get(edge_index, edge_weight, vertex_cnt, rule_cnt)
         return self.update(CooPropagateFunction.apply(plan, x))
 
+    def propagate(self, edge_index, x: Tensor, edge_weight: Optional[Tensor] = None, size: Size = None):
+        """One hop over an uncompressed graph given as a [2, E] edge tensor: out[dst] += weight * x[src]
+        (the edge-tensor branch of layer/CompressgnnPropagation.py:50-60: gather, message, scatter-add,
+        update), as one product of the HIP kernels over the edges grouped by destination, ties in edge
+        order.  The reference's other branch takes a torch_sparse SparseTensor, which this build
+        does not depend on."""
+        if not isinstance(edge_index, Tensor):
+            raise TypeError("propagate() takes a [2, E] edge tensor; compressed graphs go through compressgnn_propagate()")
+        if self.aggr not in _SUMS:
+            raise ValueError("propagate() supports aggr='add' only")
+        weights = None if edge_weight is None else [edge_weight]
+        plan = self._coo_plans.get([edge_index], weights, x.size(0), 0)
+        return self.update(CooPropagateFunction.apply(plan, x))
+
     def message(self, x_j: Tensor) -> Tensor:
         return x_j
 

@@ -701,3 +701,37 @@ def test_a_later_plan_applies_the_orders_the_first_one_found(tmp_path, monkeypat
     assert graph._plan is None
     once_more = graph.plan()
     assert torch.equal(once_more.forward(x), out) and torch.equal(once_more.backward(g), gx)
+
+
+def test_uncompressed_hop_over_an_edge_tensor():
+    """Propagate.propagate(edge_index, x, edge_weight) with a [2, E] edge tensor
+    (layer/CompressgnnPropagation.py:50-60, edge-tensor branch): out[dst] += w * x[src] in edge
+    order per destination, i.e. bit-equal to the oracle's sequential scatter-add where a
+    destination takes the row schedule; the gradient is the transposed sum; without weights every
+    edge counts 1; duplicate edges and vertices without edges included."""
+    import prep_oracle
+    from KPropagate import KPropagate
+    rng = np.random.default_rng(17)
+    V, E, F = 3000, 26000, 40
+    src = rng.integers(0, V, E)
+    dst = rng.integers(0, V - 200, E)  # the last 200 vertices receive nothing
+    src[:50], dst[:50] = src[50:100], dst[50:100]  # duplicate edges
+    w = (rng.standard_normal(E) * 0.3).astype(np.float32)
+    x_np = rng.standard_normal((V, F)).astype(np.float32)
+    edges = np.vstack((src, dst)).astype(np.int64)
+    want = prep_oracle.coo_propagate(x_np, [edges], [w], V, 0)
+    g_np = rng.standard_normal((V, F)).astype(np.float32)
+    want_gx = np.zeros_like(x_np)
+    np.add.at(want_gx, src, w.reshape(-1, 1) * g_np[dst])
+    prop = KPropagate()
+    x = torch.from_numpy(x_np).to(DEV).requires_grad_()
+    e_t, w_t = torch.from_numpy(edges).to(DEV), torch.from_numpy(w).to(DEV)
+    out = prop.propagate(e_t, x, w_t)
+    (gx,) = torch.autograd.grad(out, x, torch.from_numpy(g_np).to(DEV))
+    assert_within(out.detach().cpu().numpy(), want)
+    assert_within(gx.cpu().numpy(), want_gx, rtol=1e-5, atol=2e-6)
+    assert not out[V - 200:].any()
+    ones = prop.propagate(e_t, x)
+    assert_within(ones.detach().cpu().numpy(), prep_oracle.coo_propagate(x_np, [edges], [np.ones(E, np.float32)], V, 0))
+    with pytest.raises(TypeError):
+        prop.propagate([e_t], x, w_t)
