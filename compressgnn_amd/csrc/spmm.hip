@@ -209,6 +209,7 @@ template <typename T, int VEC, int TILES, int MODE>
 __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_t foff[TILES],
                                           const Acc<T, VEC, TILES, MODE> &acc, int accumulate) {
     T *yrow = Y + (int64_t)row * F;
+    if constexpr (MODE == MODE_DUAL) accumulate = 0;  // the two-source product writes every row once: no load on this path
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
         if (foff[t] < 0) continue;
@@ -238,10 +239,11 @@ __device__ __forceinline__ Pack<T, VEC> gather(const SpmmArgs<T> &a, int c, int 
     }
     const T *base = a.X;
     if constexpr (MODE == MODE_DUAL) {
-        if (src) {
-            base = a.X1;
-            c -= a.split;
-        }
+        // both pointers are read first and chosen between as values (a choice between the two
+        // fields of the argument block becomes a vector load of the chosen field, and a wait)
+        const T *first = a.X, *second = a.X1;
+        base = src ? second : first;
+        c -= src ? a.split : 0;
     }
     const int64_t off = (int64_t)c * (int32_t)a.F + foff;  // F < 2^31: one 32 x 32 -> 64 bit multiply
     // rows that are gathered once (member lists; masks exist for those only) are not kept in the caches
@@ -448,9 +450,13 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
     int cur = -1;
     bool continues = false;
     if (active) {
-        cur = a.rowidx[e0];
-        // asked for now, beside the entries, and looked at when the run is done
-        const int row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
+        // A run names its rows by the row of Y they are written to (rowmap[stored row], which the
+        // lanes look up beside their entries), so that closing a row inside the run needs no load
+        // of its own: a load there, and the wait for it, would stand between the gathers of the run.
+        int cur_out;
+        // looked at when the run is done: the stored row of the last entry (the row a carry belongs
+        // to) and the row of the entry behind the run; asked for beside the entries
+        int last_row, row_behind;
         if constexpr (LPR >= kUnroll && sizeof(T) == 4) {
             // As in the row schedule: the lanes of the group load one entry each, and the
             // entries reach all lanes through the LDS crossbar.
@@ -459,21 +465,28 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
 #pragma unroll
             for (int t = 0; t < TILES; ++t) fld[t] = foff[t] < 0 ? 0 : foff[t];
             for (int e = e0; e < e1; e += LPR) {
-                int my_r = 0, my_c = 0;
+                int my_o = 0, my_c = 0;
                 T my_w = T(1);
                 if (e + lane < e1) {
-                    my_r = a.rowidx[e + lane];
+                    my_o = out_row(a, a.rowidx[e + lane]);
                     my_c = a.colidx[e + lane];
                     if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) my_w = a.val[e + lane];
                 }
+                // with every batch of entries, so that no load of the run waits for another but
+                // the row numbers for their rows (the same two words each time)
+                last_row = a.rowidx[e1 - 1];
+                row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
+                // the run begins with the row of its first entry
+                const int batch_first = __builtin_amdgcn_ds_bpermute(group_lane0, my_o);
+                if (e == e0) cur_out = batch_first;
                 const int cnt = min(e1 - e, LPR);
                 for (int u0 = 0; u0 < cnt; u0 += kUnroll) {
-                    int r[kUnroll], c[kUnroll];
+                    int o[kUnroll], c[kUnroll];
                     T w[kUnroll];
 #pragma unroll
                     for (int u = 0; u < kUnroll; ++u) {
                         const int from = group_lane0 + 4 * (u0 + u);
-                        r[u] = __builtin_amdgcn_ds_bpermute(from, my_r);
+                        o[u] = __builtin_amdgcn_ds_bpermute(from, my_o);
                         c[u] = __builtin_amdgcn_ds_bpermute(from, my_c);
                         if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL)
                             w[u] = __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, my_w)));
@@ -498,11 +511,11 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u) {
                             if (u0 + u < cnt) {
-                                if (r[u] != cur) {
-                                    // row `cur` ends inside this run: finish it here
-                                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+                                if (o[u] != cur_out) {
+                                    // the row ends inside this run: finish it here
+                                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur_out, foff, acc, a.accumulate);
                                     acc.clear();
-                                    cur = r[u];
+                                    cur_out = o[u];
                                 }
                                 acc.add(x[u], w[u], kPlain ? 0 : c[u] >= a.split);
                             }
@@ -513,14 +526,17 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                 }
             }
         } else {
+            cur_out = out_row(a, a.rowidx[e0]);
+            last_row = a.rowidx[e1 - 1];
+            row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
             for (int e = e0; e < e1; e += kUnroll) {
-                int r[kUnroll], c[kUnroll];
+                int o[kUnroll], c[kUnroll];
                 T w[kUnroll];
                 Pack<T, VEC> x[kUnroll][TILES];
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u) {
                     const int idx = min(e + u, e1 - 1);
-                    r[u] = a.rowidx[idx];
+                    o[u] = out_row(a, a.rowidx[idx]);
                     c[u] = a.colidx[idx];
                     if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
                     else w[u] = T(1);
@@ -535,19 +551,20 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u) {
                     if (e + u < e1) {
-                        if (r[u] != cur) {
-                            // row `cur` ends inside this run: finish it here
-                            write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+                        if (o[u] != cur_out) {
+                            // the row ends inside this run: finish it here
+                            write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur_out, foff, acc, a.accumulate);
                             acc.clear();
-                            cur = r[u];
+                            cur_out = o[u];
                         }
                         acc.add(x[u], w[u], c[u] >= a.split);
                     }
                 }
             }
         }
+        cur = last_row;
         continues = row_behind == cur;
-        if (!continues) write_row<T, VEC, TILES, MODE>(a.Y, a.F, out_row(a, cur), foff, acc, a.accumulate);
+        if (!continues) write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur_out, foff, acc, a.accumulate);
     }
     // The carries of one row are added per workgroup: the first of its lane groups that
     // carries the row takes those of the groups behind it, in ascending order.
