@@ -493,21 +493,23 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                         else
                             w[u] = T(1);
                     }
+                    // Lanes without an entry hold column 0 (a row of X like any other) and value 1, and
+                    // positions behind the last entry of a batch read those: a round may gather for them,
+                    // nothing is added for them.  Only a block without first-source columns sees such a
+                    // position as one of the second source, and takes the slower path for that round.
                     bool second = false;
                     if constexpr (MODE == MODE_DUAL) {
 #pragma unroll
-                        for (int u = 0; u < kUnroll; ++u) second = second || (u0 + u < cnt && c[u] >= a.split);
+                        for (int u = 0; u < kUnroll; ++u) second = second | (c[u] >= a.split);
                     }
                     auto gather_and_add = [&](auto plain) {
                         constexpr bool kPlain = decltype(plain)::value;  // every entry from the first source
                         Pack<T, VEC> x[kUnroll][TILES];
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u)
-                            if (u0 + u < cnt) {
 #pragma unroll
-                                for (int t = 0; t < TILES; ++t)
-                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
-                            }
+                            for (int t = 0; t < TILES; ++t)
+                                x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u) {
                             if (u0 + u < cnt) {
