@@ -209,7 +209,10 @@ template <typename T, int VEC, int TILES, int MODE>
 __device__ __forceinline__ void write_row(T *Y, int64_t F, int row, const int64_t foff[TILES],
                                           const Acc<T, VEC, TILES, MODE> &acc, int accumulate) {
     T *yrow = Y + (int64_t)row * F;
-    if constexpr (MODE == MODE_DUAL) accumulate = 0;  // the two-source product writes every row once: no load on this path
+    // Only the plain product (MODE_VAL) can add to an existing Y.  The other modes write every row once, and
+    // knowing that at compile time keeps a load of Y out of the block that closes a row inside a run of the
+    // nnz schedule, where the compiler would have to wait for it on every path behind the block.
+    if constexpr (MODE != MODE_VAL) accumulate = 0;
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
         if (foff[t] < 0) continue;
@@ -470,7 +473,8 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                 if (e + lane < e1) {
                     my_o = out_row(a, a.rowidx[e + lane]);
                     my_c = a.colidx[e + lane];
-                    if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) my_w = a.val[e + lane];
+                    if constexpr (MODE == MODE_DUAL) my_w = a.val[e + lane];
+                    if constexpr (MODE == MODE_VAL) my_w = a.val != nullptr ? a.val[e + lane] : T(1);
                 }
                 // with every batch of entries, so that no load of the run waits for another but
                 // the row numbers for their rows (the same two words each time)
@@ -540,7 +544,8 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                     const int idx = min(e + u, e1 - 1);
                     o[u] = out_row(a, a.rowidx[idx]);
                     c[u] = a.colidx[idx];
-                    if constexpr (MODE == MODE_VAL || MODE == MODE_DUAL) w[u] = a.val[idx];
+                    if constexpr (MODE == MODE_DUAL) w[u] = a.val[idx];
+                    else if constexpr (MODE == MODE_VAL) w[u] = a.val != nullptr ? a.val[idx] : T(1);
                     else w[u] = T(1);
                 }
 #pragma unroll
@@ -1118,7 +1123,8 @@ int spmm_typed(const cgnn_csr *A, const void *X, const void *X1, int64_t split, 
     }
     kernel = resolve_kernel(A, kernel);
     if (masked) kernel = CGNN_SPMM_NNZ;  // masks exist for the nnz schedule only
-    if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ) mode = MODE_UNIT;
+    // unit values without the multiplications; a product that adds to Y stays with the plain mode, the only one that reads Y
+    if (mode == MODE_VAL && A->val == nullptr && kernel == CGNN_SPMM_NNZ && !accumulate) mode = MODE_UNIT;
     if (mode == MODE_DUAL && A->nnz > 0 && A->val == nullptr)
         return fail(CGNN_EINVAL, "spmm: the two-source product needs stored values");
     if (kernel == CGNN_SPMM_ROW) {

@@ -400,3 +400,29 @@ def test_table_of_run_starts(seg, F):
     again = B.spmm(X, None, "nnz_schedule")
     assert B.run_start.numel() == (nnz + 2 * K - 1) // (2 * K) + 1
     assert_within(again.cpu().numpy(), oracle.spmm(vlist, elist, value, x))
+
+
+@pytest.mark.parametrize("kernel", [abi.SPMM_ROW, abi.SPMM_NNZ])
+@pytest.mark.parametrize("F", [16, 100, 128])
+def test_blocks_without_stored_values(kernel, F):
+    """val == NULL stands for ones (the ABI's convention; member lists are such blocks): fresh and
+    accumulating products in both schedules against the oracle with explicit ones.  Additions of
+    x * 1 and of x are the same additions, so rows that no run cuts keep the oracle's bits."""
+    rng = np.random.default_rng(31 + F)
+    rows, cols = 900, 500
+    vlist, elist, _ = random_csr(rng, rows, cols, 5.0, skew=True)
+    ones = np.ones(len(elist), np.float32)
+    x = (rng.standard_normal((cols, F)) * 0.1).astype(np.float32)
+    out0 = rng.standard_normal((rows, F)).astype(np.float32)
+    A = abi.DeviceCsr.from_host(rows, cols, vlist, elist, None, DEV, seg_nnz=32)
+    X = torch.from_numpy(x).to(DEV)
+    fresh = abi.spmm(A, X, None, False, kernel).cpu().numpy()
+    acc = abi.spmm(A, X, torch.from_numpy(out0.copy()).to(DEV), True, kernel).cpu().numpy()
+    want, want_acc = oracle.spmm(vlist, elist, ones, x), oracle.spmm(vlist, elist, ones, x, out0.copy())
+    # unit weights on rows of up to thousands of entries: cut rows re-associate beyond 1e-6 absolute
+    assert_within(fresh, want, rtol=1e-5, atol=2e-5)
+    assert_within(acc, want_acc, rtol=1e-5, atol=2e-5)
+    whole = np.diff(vlist) <= 32 if kernel == abi.SPMM_NNZ else np.ones(rows, bool)
+    assert np.array_equal(fresh[whole], want[whole]) and np.array_equal(acc[whole], want_acc[whole])
+    empty = np.diff(vlist) == 0
+    assert np.array_equal(acc[empty], out0[empty]) and not fresh[empty].any()
