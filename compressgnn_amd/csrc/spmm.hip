@@ -456,10 +456,24 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
         // A run names its rows by the row of Y they are written to (rowmap[stored row], which the
         // lanes look up beside their entries), so that closing a row inside the run needs no load
         // of its own: a load there, and the wait for it, would stand between the gathers of the run.
+        // The two-source product over rows of 512 bytes and more keeps the other form -- the run names
+        // its rows by their stored number and looks the row of Y up where a row ends.  The look-up
+        // beside the entries puts one more load between a run's entries and its first gathers and
+        // holds two more values per lane in a kernel that sits at its register limit (72 for seven
+        // waves per SIMD): the F = 128 kernel, bound by its traffic either way, took 221 us with it
+        // and takes 213 us without (F = 16: 76 -> 62 us with it; the 18.5 M-vertex graph at F = 64:
+        // 13.6 -> 13.4 ms; the mask modes, which have no rowmap, lose the wait and nothing else).
+        constexpr bool kNamesRowsOfY = !(MODE == MODE_DUAL && VEC * LPR * sizeof(T) >= 512);
+        auto named = [&](int stored_row) { return kNamesRowsOfY ? out_row(a, stored_row) : stored_row; };
+        auto row_of_y = [&](int name) { return kNamesRowsOfY ? name : out_row(a, name); };
         int cur_out;
         // looked at when the run is done: the stored row of the last entry (the row a carry belongs
         // to) and the row of the entry behind the run; asked for beside the entries
         int last_row, row_behind;
+        if constexpr (!kNamesRowsOfY) {  // the names are the stored rows: the first is read here, the last is at hand at the end
+            cur_out = a.rowidx[e0];
+            row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
+        }
         if constexpr (LPR >= kUnroll && sizeof(T) == 4) {
             // As in the row schedule: the lanes of the group load one entry each, and the
             // entries reach all lanes through the LDS crossbar.
@@ -471,18 +485,20 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                 int my_o = 0, my_c = 0;
                 T my_w = T(1);
                 if (e + lane < e1) {
-                    my_o = out_row(a, a.rowidx[e + lane]);
+                    my_o = named(a.rowidx[e + lane]);
                     my_c = a.colidx[e + lane];
                     if constexpr (MODE == MODE_DUAL) my_w = a.val[e + lane];
                     if constexpr (MODE == MODE_VAL) my_w = a.val != nullptr ? a.val[e + lane] : T(1);
                 }
-                // with every batch of entries, so that no load of the run waits for another but
-                // the row numbers for their rows (the same two words each time)
-                last_row = a.rowidx[e1 - 1];
-                row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
-                // the run begins with the row of its first entry
-                const int batch_first = __builtin_amdgcn_ds_bpermute(group_lane0, my_o);
-                if (e == e0) cur_out = batch_first;
+                if constexpr (kNamesRowsOfY) {
+                    // with every batch of entries, so that no load of the run waits for another but
+                    // the row numbers for their rows (the same two words each time)
+                    last_row = a.rowidx[e1 - 1];
+                    row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
+                    // the run begins with the row of its first entry
+                    const int batch_first = __builtin_amdgcn_ds_bpermute(group_lane0, my_o);
+                    if (e == e0) cur_out = batch_first;
+                }
                 const int cnt = min(e1 - e, LPR);
                 for (int u0 = 0; u0 < cnt; u0 += kUnroll) {
                     int o[kUnroll], c[kUnroll];
@@ -509,17 +525,23 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                     auto gather_and_add = [&](auto plain) {
                         constexpr bool kPlain = decltype(plain)::value;  // every entry from the first source
                         Pack<T, VEC> x[kUnroll][TILES];
+                        // Up to 64 bytes per lane group and gather, a position behind the last entry gathers
+                        // like the others (column 0, see above): the branches around four small loads cost
+                        // more than the loads.  Wider rows skip it: there the extra row is what costs.
+                        constexpr bool kGatherAll = VEC * LPR * sizeof(T) <= 64;
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u)
+                            if (kGatherAll || u0 + u < cnt) {
 #pragma unroll
-                            for (int t = 0; t < TILES; ++t)
-                                x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
+                                for (int t = 0; t < TILES; ++t)
+                                    x[u][t] = gather<T, VEC, MODE>(a, c[u], kPlain ? 0 : c[u] >= a.split, fld[t]);
+                            }
 #pragma unroll
                         for (int u = 0; u < kUnroll; ++u) {
                             if (u0 + u < cnt) {
                                 if (o[u] != cur_out) {
                                     // the row ends inside this run: finish it here
-                                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur_out, foff, acc, a.accumulate);
+                                    write_row<T, VEC, TILES, MODE>(a.Y, a.F, row_of_y(cur_out), foff, acc, a.accumulate);
                                     acc.clear();
                                     cur_out = o[u];
                                 }
@@ -532,9 +554,11 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                 }
             }
         } else {
-            cur_out = out_row(a, a.rowidx[e0]);
-            last_row = a.rowidx[e1 - 1];
-            row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
+            if constexpr (kNamesRowsOfY) {
+                cur_out = named(a.rowidx[e0]);
+                last_row = a.rowidx[e1 - 1];
+                row_behind = e1 < a.nnz ? a.rowidx[e1] : -1;
+            }
             for (int e = e0; e < e1; e += kUnroll) {
                 int o[kUnroll], c[kUnroll];
                 T w[kUnroll];
@@ -542,7 +566,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u) {
                     const int idx = min(e + u, e1 - 1);
-                    o[u] = out_row(a, a.rowidx[idx]);
+                    o[u] = named(a.rowidx[idx]);
                     c[u] = a.colidx[idx];
                     if constexpr (MODE == MODE_DUAL) w[u] = a.val[idx];
                     else if constexpr (MODE == MODE_VAL) w[u] = a.val != nullptr ? a.val[idx] : T(1);
@@ -560,7 +584,7 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                     if (e + u < e1) {
                         if (o[u] != cur_out) {
                             // the row ends inside this run: finish it here
-                            write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur_out, foff, acc, a.accumulate);
+                            write_row<T, VEC, TILES, MODE>(a.Y, a.F, row_of_y(cur_out), foff, acc, a.accumulate);
                             acc.clear();
                             cur_out = o[u];
                         }
@@ -569,9 +593,9 @@ __global__ __launch_bounds__(kBlock, (TILES == 1 && LPR >= 16) ? 7 : 1) void spm
                 }
             }
         }
-        cur = last_row;
+        cur = kNamesRowsOfY ? last_row : cur_out;
         continues = row_behind == cur;
-        if (!continues) write_row<T, VEC, TILES, MODE>(a.Y, a.F, cur_out, foff, acc, a.accumulate);
+        if (!continues) write_row<T, VEC, TILES, MODE>(a.Y, a.F, row_of_y(cur_out), foff, acc, a.accumulate);
     }
     // The carries of one row are added per workgroup: the first of its lane groups that
     // carries the row takes those of the groups behind it, in ascending order.
