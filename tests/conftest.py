@@ -4,7 +4,11 @@ import sys
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-for p in (ROOT, os.path.join(ROOT, "oracle"), os.path.join(ROOT, "oracle", "_ref")):
+# the package's modules are imported by bare name, as the reference's scripts import its layers
+# (model/compressgnn/gcn.py:3-8): every test file finds them, run alone or with the others
+PACKAGE = os.path.join(ROOT, "compressgnn_amd")
+for p in (ROOT, os.path.join(ROOT, "oracle"), os.path.join(ROOT, "oracle", "_ref"), PACKAGE,
+          os.path.join(PACKAGE, "layer"), os.path.join(PACKAGE, "loader"), os.path.dirname(os.path.abspath(__file__))):
     if p not in sys.path:
         sys.path.insert(0, p)
 
