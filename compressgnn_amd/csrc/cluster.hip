@@ -370,7 +370,12 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_mfma_kernel(LshArgs<float> 
 // a wave-uniform condition.  The code of a tile is stored (and its bucket counted) only
 // after the next tile has been committed to LDS, so that no wait for the loads also waits
 // for that atomic.
+//
+// The tiles of a workgroup (those a static deal would give its waves) are handed out by a
+// counter in LDS, one at a time: six waves on four SIMDs means two SIMDs carry two waves
+// and two carry one, and a wave that has a SIMD to itself gets through its tiles faster.
 constexpr int kLshFlatMaxWaves = 8;
+constexpr int kLshQueueBytes = 16;  // the counter, padded so that the tiles stay 16-byte aligned
 
 template <int NG, int XP>
 __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat_kernel(LshArgs<float> a,
@@ -382,12 +387,14 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
     const int wave = threadIdx.x / kLshRows;
     const int waves = blockDim.x / kLshRows;
     float *wtile = reinterpret_cast<float *>(lds_raw);
-    lsh_f4_t *tile = reinterpret_cast<lsh_f4_t *>(lds_raw + (size_t)a.wstride * 16 * NG * sizeof(float)) +
+    const size_t plane_bytes = (size_t)a.wstride * 16 * NG * sizeof(float);
+    int *queue = reinterpret_cast<int *>(lds_raw + plane_bytes);
+    lsh_f4_t *tile = reinterpret_cast<lsh_f4_t *>(lds_raw + plane_bytes + kLshQueueBytes) +
                      (size_t)wave * kLshRows * a.stride_v;
     const int H = a.bits;
     const int ks_v = a.F / 4;  // packs per row = packs per lane and tile
     const lsh_f4_t *X4 = reinterpret_cast<const lsh_f4_t *>(a.X);
-    const int64_t first = (int64_t)blockIdx.x * waves + wave;
+    const int64_t first = (int64_t)blockIdx.x * waves;
     const int64_t step = (int64_t)gridDim.x * waves;
     const GlobalSink sink{a.bucket_count};
 
@@ -395,7 +402,16 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
         const int kk = e / (16 * NG), j = e % (16 * NG);
         wtile[j * a.wstride + kk] = j < H ? a.W[(int64_t)kk * H + j] : 0.f;
     }
+    if (threadIdx.x == 0) *queue = 0;
     __syncthreads();
+    // the j-th tile of this workgroup; grows with j, so a wave that draws one beyond the
+    // end is done, and so is every later draw
+    auto take = [&]() -> int64_t {
+        int j = 0;
+        if (lane == 0) j = atomicAdd(queue, 1);
+        j = __builtin_amdgcn_readfirstlane(j);
+        return (int64_t)(j / waves) * step + first + j % waves;
+    };
 
     lsh_acc_t acc[NG];
 #pragma unroll
@@ -428,6 +444,9 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
 #pragma unroll
             for (int g = 0; g < NG; ++g) w[g][i] = wq[g * gstep + c + i];
         }
+        // left to itself the scheduler sinks every pair of reads to its four matrix
+        // instructions, into one set of registers, and pays the LDS latency per pack
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < n; ++i)
 #pragma unroll
@@ -440,8 +459,9 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
     WaveCodeCounter counter;
     int pending_code = 0;
     int64_t pending_row = -1;
-    if (first < tiles) fetch(first);
-    for (int64_t t = first; t < tiles; t += step) {
+    int64_t t = take();
+    if (t < tiles) fetch(t);
+    while (t < tiles) {
         wave_lds_sync();  // the previous tile has been consumed
 #pragma unroll
         for (int u = 0; u < XP; ++u) {
@@ -451,7 +471,8 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
         wave_lds_sync();
         if (pending_row >= 0 && pending_row < a.N) a.raw_code[pending_row] = pending_code;
         if (a.bucket_count != nullptr) counter.add(sink, pending_code, pending_row >= 0 && pending_row < a.N, lane);
-        if (t + step < tiles) fetch(t + step);
+        const int64_t t_next = take();
+        if (t_next < tiles) fetch(t_next);
 
         // eight column packs at a time: all sixteen LDS reads are issued before the first
         // multiply, so their latency is paid once per 32 matrix instructions
@@ -478,6 +499,7 @@ __global__ __launch_bounds__(kLshRows *kLshFlatMaxWaves) void lsh_hash_mfma_flat
         if (NG == 2) mask |= ((uint32_t)(sel[NG - 1] >> shift) & 0xffffu) << 16;
         pending_code = (int)(__brev(mask) >> (32 - H));  // plane 0 is the top bit
         pending_row = t * kLshRows + lane;
+        t = t_next;
     }
     if (pending_row >= 0 && pending_row < a.N) a.raw_code[pending_row] = pending_code;
     if (a.bucket_count != nullptr) counter.add(sink, pending_code, pending_row >= 0 && pending_row < a.N, lane);
@@ -551,7 +573,7 @@ int launch_lsh_flat(const LshArgs<float> &a, hipStream_t stream) {
     const size_t tile_bytes = (size_t)kLshRows * a.stride_v * sizeof(lsh_f4_t);
     const size_t plane_bytes = (size_t)a.wstride * 16 * NG * sizeof(float);
     // as many waves as fit beside one copy of the planes; two per SIMD at most (registers)
-    const size_t fixed_bytes = plane_bytes;
+    const size_t fixed_bytes = plane_bytes + kLshQueueBytes;
     int waves = (int)((kLdsPerCu - fixed_bytes) / tile_bytes);
     waves = waves < 1 ? 1 : (waves > kLshFlatMaxWaves ? kLshFlatMaxWaves : waves);
     auto kernel = lsh_hash_mfma_flat_kernel<NG, XP>;
