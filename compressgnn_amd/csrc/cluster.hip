@@ -195,7 +195,8 @@ __global__ __launch_bounds__(kLshRows) void lsh_hash_kernel(LshArgs<T> a) {
 // A pass stages up to 128 columns of the 64 rows, so rows of up to 512 bytes are read
 // whole and every cache line of X is fetched once.  That much LDS per wave leaves room for
 // only a few waves per compute unit, so the waves are persistent (each walks tiles
-// t, t + stride, ...) and keep the next pass in registers, in flight, while they multiply
+// t, t + stride, ... in the general form; in the flat form a workgroup's waves draw from
+// its tiles in turn) and keep the next pass in registers, in flight, while they multiply
 // the current one out of LDS.  W is staged with zero columns beyond `bits`; NG = 2 covers
 // 17..30 planes with two instructions per k.  lsh_hash_mfma_kernel is the general form
 // (any F, several passes per tile); lsh_hash_mfma_flat_kernel below is the form for
