@@ -31,25 +31,40 @@ static_assert(kDigits == kBlock, "one digit per thread");
 __device__ __forceinline__ int digit_of(int32_t key, int shift) { return (key >> shift) & (kDigits - 1); }
 
 // hist[d * tiles + tile] = number of keys of the tile with digit d (digit-major: the scan over a
-// digit's tiles is a scan over consecutive entries).  `clear` (optional, first pass): a table of
-// clear_n entries that this launch sets to zero, for the scatter of the same pass to mark.
+// digit's tiles is a scan over consecutive entries).  THREADS: the workgroup's size, a multiple
+// of kDigits; the loads of a thread are all issued before the first count.
+template <int THREADS>
+__device__ __forceinline__ void tile_histogram(const int32_t *__restrict__ keys, int64_t N, int shift,
+                                               int32_t *__restrict__ hist, int tiles, int tile, int *count) {
+    constexpr int kItems = kSortTile / THREADS;
+    if (threadIdx.x < kDigits) count[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)tile * kSortTile;
+    int32_t key[kItems];
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) {
+        const int64_t i = base + (int64_t)it * THREADS + threadIdx.x;
+        key[it] = i < N ? keys[i] : 0;
+    }
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) {
+        const int64_t i = base + (int64_t)it * THREADS + threadIdx.x;
+        if (i < N) atomicAdd(&count[digit_of(key[it], shift)], 1);  // LDS, integer: the sum does not depend on the order
+    }
+    __syncthreads();
+    if (threadIdx.x < kDigits) hist[(int64_t)threadIdx.x * tiles + tile] = count[threadIdx.x];
+}
+
+// `clear` (optional, first pass): a table of clear_n entries that this launch sets to zero, for
+// the scatter of the same pass to mark.
 __global__ __launch_bounds__(kBlock) void radix_hist_kernel(const int32_t *__restrict__ keys, int64_t N, int shift,
                                                            int32_t *__restrict__ hist, int tiles,
                                                            int32_t *__restrict__ clear, int clear_n) {
     __shared__ int count[kDigits];
-    count[threadIdx.x] = 0;
     if (clear)
         for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < clear_n; i += (int64_t)gridDim.x * kBlock)
             clear[i] = 0;
-    __syncthreads();
-    const int64_t base = (int64_t)blockIdx.x * kSortTile;
-#pragma unroll
-    for (int it = 0; it < kSortItems; ++it) {
-        const int64_t i = base + (int64_t)it * kBlock + threadIdx.x;
-        if (i < N) atomicAdd(&count[digit_of(keys[i], shift)], 1);  // LDS, integer: the sum does not depend on the order
-    }
-    __syncthreads();
-    hist[(int64_t)threadIdx.x * tiles + blockIdx.x] = count[threadIdx.x];
+    tile_histogram<kBlock>(keys, N, shift, hist, tiles, blockIdx.x, count);
 }
 
 // One wave per digit: within[d * tiles + t] = keys with digit d in the tiles before t, and
@@ -288,10 +303,12 @@ constexpr int kRankStretches = (1 << kTableBits) / kRankStretch;
 
 __device__ __forceinline__ int occurs4(const int4 &v) { return (v.x != 0) + (v.y != 0) + (v.z != 0) + (v.w != 0); }
 
-__global__ __launch_bounds__(kRankThreads) void code_rank_kernel(int32_t *__restrict__ table, int codes,
-                                                                 int32_t *__restrict__ summary) {
-    constexpr int kWaves = kRankThreads / kWave;
-    __shared__ int wave_before[kWaves], wave_mine[kWaves];
+constexpr int kRankWaves = kRankThreads / kWave;
+
+// stretch `part` of `parts`
+__device__ __forceinline__ void code_rank_stretch(int32_t *__restrict__ table, int codes, int32_t *__restrict__ summary,
+                                                  int part, int parts, int *wave_before, int *wave_mine) {
+    constexpr int kWaves = kRankWaves;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int4 *table4 = reinterpret_cast<const int4 *>(table);  // codes is a power of two: whole int4s from 4 codes on
     const int4 zero = {0, 0, 0, 0};
@@ -301,9 +318,9 @@ __global__ __launch_bounds__(kRankThreads) void code_rank_kernel(int32_t *__rest
 #pragma unroll
     for (int k = 0; k < kRankStretches - 1; ++k) {
         const int q = k * kRankThreads + threadIdx.x;
-        earlier[k] = (k < (int)blockIdx.x && q < quads && codes >= 4) ? table4[q] : zero;
+        earlier[k] = (k < part && q < quads && codes >= 4) ? table4[q] : zero;
     }
-    const int q = blockIdx.x * kRankThreads + threadIdx.x;
+    const int q = part * kRankThreads + threadIdx.x;
     int4 own = zero;
     if (codes >= 4) {
         if (q < quads) own = table4[q];
@@ -345,10 +362,32 @@ __global__ __launch_bounds__(kRankThreads) void code_rank_kernel(int32_t *__rest
         table[0] = out.x;
         if (codes > 1) table[1] = out.y;
     }
-    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+    if (part == parts - 1 && threadIdx.x == 0) {
         summary[0] = stretch_total;
         summary[1] = 0;
     }
+}
+
+__global__ __launch_bounds__(kRankThreads) void code_rank_kernel(int32_t *__restrict__ table, int codes,
+                                                                 int32_t *__restrict__ summary) {
+    __shared__ int wave_before[kRankWaves], wave_mine[kRankWaves];
+    code_rank_stretch(table, codes, summary, blockIdx.x, gridDim.x, wave_before, wave_mine);
+}
+
+// The histograms of a later pass and the ranks of the codes in one launch: neither needs the
+// other, both need the scatter of the first pass (its keys; the codes it has marked), and the
+// sixteen workgroups of the ranks are over before the histograms are.
+__global__ __launch_bounds__(kRankThreads) void radix_hist_rank_kernel(const int32_t *__restrict__ keys, int64_t N,
+                                                                       int shift, int32_t *__restrict__ hist, int tiles,
+                                                                       int32_t *__restrict__ table, int codes,
+                                                                       int32_t *__restrict__ summary) {
+    __shared__ int count[kDigits];
+    __shared__ int wave_before[kRankWaves], wave_mine[kRankWaves];
+    const int parts = (int)gridDim.x - tiles;
+    if ((int)blockIdx.x < parts)  // first, so that they are not the tail of the launch
+        code_rank_stretch(table, codes, summary, blockIdx.x, parts, wave_before, wave_mine);
+    else
+        tile_histogram<kRankThreads>(keys, N, shift, hist, tiles, (int)blockIdx.x - parts, count);
 }
 
 // Stable sort of (keys[i], i) by the low `bits` bits of the keys into (keys_out, vals_out).
@@ -377,15 +416,21 @@ int radix_sort_by_key(const int32_t *keys, int64_t N, int bits, int32_t *keys_ou
         const int shift = p * kDigitBits;
         const bool first = p == 0, last = p == passes - 1;
         const int32_t *remap = (table && last && !first) ? table : nullptr;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, in_keys, N, shift, hist,
-                           tiles, first ? table : nullptr, seen_mask + 1);
+        const int rank_parts = (int)ceil_div(seen_mask + 1, kRankStretch);
+        const bool rank_here = table && p == 1;  // the marks are complete after the first scatter
+        if (rank_here)
+            hipLaunchKernelGGL(radix_hist_rank_kernel, dim3((unsigned)(tiles + rank_parts)), dim3(kRankThreads), 0,
+                               stream, in_keys, N, shift, hist, tiles, table, seen_mask + 1, summary);
+        else
+            hipLaunchKernelGGL(radix_hist_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, in_keys, N, shift,
+                               hist, tiles, first ? table : nullptr, seen_mask + 1);
         hipLaunchKernelGGL(radix_scan_kernel, dim3(kDigits / (kBlock / kWave)), dim3(kBlock), 0, stream, hist, tiles,
                            within, total);
         hipLaunchKernelGGL(radix_scatter_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, in_keys, in_vals, N,
                            shift, within, total, tiles, out_keys, out_vals, first ? table : nullptr, seen_mask, remap);
-        if (table && first)
-            hipLaunchKernelGGL(code_rank_kernel, dim3((unsigned)ceil_div(seen_mask + 1, kRankStretch)), dim3(kRankThreads),
-                               0, stream, table, seen_mask + 1, summary);
+        if (table && first && last)  // with a second pass its histogram launch makes the ranks
+            hipLaunchKernelGGL(code_rank_kernel, dim3((unsigned)rank_parts), dim3(kRankThreads), 0, stream, table,
+                               seen_mask + 1, summary);
         if (remap && ranked) *ranked = true;
         in_keys = out_keys;
         in_vals = out_vals;
@@ -401,18 +446,39 @@ __global__ __launch_bounds__(kBlock) void group_table_finish_kernel(int64_t N, c
                                                                    const int32_t *__restrict__ rank, int code_mask,
                                                                    bool ranked, int64_t *__restrict__ ids,
                                                                    int32_t *sorted_id, int32_t *__restrict__ offsets) {
-    for (int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x; p < N; p += (int64_t)gridDim.x * kBlock) {
-        ids[p] = rank[raw_code[p] & code_mask];
-        const int32_t here = sorted[p];
-        const int32_t id = ranked ? here : rank[here & code_mask];
-        if (!ranked) sorted_id[p] = id;
-        if (p == 0) {
-            offsets[0] = 0;
-            offsets[id] = 0;
-        } else if (here != sorted[p - 1]) {  // codes and their ranks change at the same places
-            offsets[id] = (int32_t)p;
+    // four positions a thread, a launch-wide stride apart: their loads are in flight together
+    constexpr int kFinishItems = 4;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t p0 = (int64_t)blockIdx.x * kBlock + threadIdx.x; p0 < N; p0 += kFinishItems * stride) {
+        int32_t code[kFinishItems], here[kFinishItems], before[kFinishItems];
+#pragma unroll
+        for (int u = 0; u < kFinishItems; ++u) {
+            const int64_t p = p0 + u * stride;
+            const bool live = p < N;
+            code[u] = live ? raw_code[p] : 0;
+            here[u] = live ? sorted[p] : 0;
+            before[u] = live && p > 0 ? sorted[p - 1] : 0;
         }
-        if (p == N - 1) offsets[id + 1] = (int32_t)N;
+        int32_t own_id[kFinishItems], id[kFinishItems];
+#pragma unroll
+        for (int u = 0; u < kFinishItems; ++u) {
+            own_id[u] = rank[code[u] & code_mask];
+            id[u] = ranked ? here[u] : rank[here[u] & code_mask];
+        }
+#pragma unroll
+        for (int u = 0; u < kFinishItems; ++u) {
+            const int64_t p = p0 + u * stride;
+            if (p >= N) continue;
+            ids[p] = own_id[u];
+            if (!ranked) sorted_id[p] = id[u];
+            if (p == 0) {
+                offsets[0] = 0;
+                offsets[id[u]] = 0;
+            } else if (here[u] != before[u]) {  // codes and their ranks change at the same places
+                offsets[id[u]] = (int32_t)p;
+            }
+            if (p == N - 1) offsets[id[u] + 1] = (int32_t)N;
+        }
     }
 }
 
@@ -529,7 +595,9 @@ extern "C" int cgnn_lsh_group(int64_t N, int bits, const int32_t *raw_code, int6
         rc = radix_sort_by_key(raw_code, N, bits, sorted, perm, tmp_keys, tmp_vals, counters, table, codes - 1, summary,
                                &ranked, stream);
         if (rc != CGNN_OK) return rc;
-        hipLaunchKernelGGL(group_table_finish_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, N, raw_code, sorted,
+        int64_t fblocks = ceil_div(N, 4 * kBlock);  // four positions a thread
+        if (fblocks > 8192) fblocks = 8192;
+        hipLaunchKernelGGL(group_table_finish_kernel, dim3((unsigned)fblocks), dim3(kBlock), 0, stream, N, raw_code, sorted,
                            table, codes - 1, ranked, ids, sorted_id, offsets);
     } else {
         int32_t *head = reinterpret_cast<int32_t *>(rest);
