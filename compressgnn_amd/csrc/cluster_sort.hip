@@ -393,7 +393,8 @@ __global__ __launch_bounds__(kRankThreads) void radix_hist_rank_kernel(const int
 // Stable sort of (keys[i], i) by the low `bits` bits of the keys into (keys_out, vals_out).
 // tmp_keys / tmp_vals: N entries each, used when there is more than one pass.  counters:
 // radix_counter_bytes(N).  table (optional): seen_mask + 1 entries (a power of two); the first
-// pass clears it and marks every key that occurs, code_rank_kernel then turns it into the ranks
+// pass clears it and marks every key that occurs, code_rank_stretch (a launch of its own after
+// a single pass, else part of the second pass's histogram launch) then turns it into the ranks
 // of the keys (summary as there), and with more than one pass the last pass writes the ranks
 // in place of the keys (*ranked = true).
 int radix_sort_by_key(const int32_t *keys, int64_t N, int bits, int32_t *keys_out, int32_t *vals_out, int32_t *tmp_keys,
