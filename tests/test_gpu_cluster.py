@@ -112,6 +112,23 @@ def test_assign_shapes(width, bits):
     assert np.array_equal(counts.cpu().numpy(), want_counts)
 
 
+@pytest.mark.parametrize("width,bits", [(100, 16), (64, 16), (128, 20)])
+def test_assign_many_tiles_a_wave(width, bits):
+    """A million rows: every wave of the projection kernel takes some six to ten tiles from
+    its workgroup's queue (six, eight and four waves a workgroup at these widths); ids and
+    counts against the oracle, bit for bit."""
+    n = 1_000_003
+    rng = np.random.default_rng(width + bits)
+    x = rng.standard_normal((n, width)).astype(np.float32)
+    w = rng.standard_normal((width, bits)).astype(np.float32)
+    want_ids, want_counts, want_active = oracle.assign(x, w, bits)
+    ids, counts, active = abi.lsh_assign(_t(x), _t(w), bits)
+    torch.cuda.synchronize()
+    assert active == want_active
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert np.array_equal(counts.cpu().numpy(), want_counts)
+
+
 @pytest.mark.parametrize("shape", ["uniform", "one_code", "few_codes", "relu"])
 @pytest.mark.parametrize("bits", [1, 8, 16, 23])
 def test_grouped_assign_matches_counter_path(shape, bits):
