@@ -871,6 +871,54 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
     }
 }
 
+// Mean gradient in natural row order over rows that are not whole cache lines: the output is
+// walked as one array of 16-byte packs, so every store instruction of a wave covers 64
+// consecutive packs -- whole 128-byte lines -- wherever the rows begin and end.  A workgroup
+// takes 64 rows (a whole number of lines whatever F is); pack l of them lies in row
+// l / packs_per_row, by multiplication (exact for l < 2^16).
+constexpr int kFlatRows = 64;
+constexpr int kFlatItems = 4;  // packs of a thread in flight together
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void mean_grad_flat_kernel(GatherArgs<T> a, int ppr, uint32_t magic) {
+    const int64_t row0 = (int64_t)blockIdx.x * kFlatRows;
+    const int rows = (int)min((int64_t)kFlatRows, a.N - row0);
+    const int packs = rows * ppr;
+    const LPack<T, VEC> *src = reinterpret_cast<const LPack<T, VEC> *>(a.src);
+    T *out = a.out + row0 * a.F;
+    for (int l0 = threadIdx.x; l0 < packs; l0 += kFlatItems * kBlock) {
+        int col[kFlatItems];
+        int64_t g[kFlatItems];
+#pragma unroll
+        for (int u = 0; u < kFlatItems; ++u) {
+            const int l = min(l0 + u * kBlock, packs - 1);
+            const int r = (int)__umulhi((uint32_t)l, magic);
+            col[u] = l - r * ppr;
+            g[u] = a.ids[row0 + r];
+        }
+        T denom[kFlatItems];
+        LPack<T, VEC> x[kFlatItems];
+#pragma unroll
+        for (int u = 0; u < kFlatItems; ++u) {
+            // an id that names no row of src is moved to the nearest row that exists and reported
+            if (g[u] < 0 || g[u] >= a.groups) {
+                g[u] = g[u] < 0 ? 0 : a.groups - 1;
+                if (a.bad_id) *a.bad_id = 1;  // every writer stores the same value
+            }
+            denom[u] = (T)max(a.counts[g[u]], 1);
+            x[u] = src[g[u] * ppr + col[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < kFlatItems; ++u) {
+            const int l = l0 + u * kBlock;
+            if (l >= packs) break;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) x[u].v[i] = x[u].v[i] / denom[u];
+            store_stream<T, VEC>(out + (int64_t)l * VEC, x[u]);
+        }
+    }
+}
+
 template <typename T, int VEC, int OP>
 int launch_gather_lpr(const GatherArgs<T> &a, hipStream_t stream) {
     const int64_t slots = a.F / VEC;
@@ -896,7 +944,20 @@ int launch_gather(const GatherArgs<T> &a, hipStream_t stream) {
         return fail(CGNN_EUNSUPPORTED, "gather: too many rows");
     constexpr int WIDE = 16 / sizeof(T);
     auto al = [](const void *p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (a.F % WIDE == 0 && al(a.src) && al(a.out) && al(a.bias)) return launch_gather_lpr<T, WIDE, OP>(a, stream);
+    const bool wide = a.F % WIDE == 0 && al(a.src) && al(a.out) && al(a.bias);
+    if constexpr (OP == GATHER_MEAN_GRAD) {
+        const int64_t ppr = a.F / WIDE;
+        if (wide && a.perm == nullptr && (a.F * (int64_t)sizeof(T)) % 128 != 0 && kFlatRows * ppr < (1 << 16) &&
+            ceil_div(a.N, kFlatRows) < ((int64_t)1 << 31)) {
+            const uint32_t magic = ppr > 1 ? (uint32_t)((1ull << 32) / (uint32_t)ppr) + 1u : 0u;
+            if (ppr > 1) {
+                hipLaunchKernelGGL((mean_grad_flat_kernel<T, WIDE>), dim3((unsigned)ceil_div(a.N, kFlatRows)), dim3(kBlock),
+                                   0, stream, a, (int)ppr, magic);
+                return check_launch("mean_grad_flat");
+            }
+        }
+    }
+    if (wide) return launch_gather_lpr<T, WIDE, OP>(a, stream);
     return launch_gather_lpr<T, 1, OP>(a, stream);
 }
 
