@@ -871,18 +871,20 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(GatherArgs<T> a) {
     }
 }
 
-// Mean gradient in natural row order over rows that are not whole cache lines: the output is
-// walked as one array of 16-byte packs, so every store instruction of a wave covers 64
+// Both gathers in natural row order over rows that are not whole cache lines (and, for the
+// reconstruct, without sign words): the output is walked as one array of 16-byte packs, so every store instruction of a wave covers 64
 // consecutive packs -- whole 128-byte lines -- wherever the rows begin and end.  A workgroup
-// takes 64 rows (a whole number of lines whatever F is); pack l of them lies in row
-// l / packs_per_row, by multiplication (exact for l < 2^16).
+// takes a multiple of 64 rows (a whole number of lines whatever F is), enough of them for
+// every thread to have four packs; pack l of them lies in row l / packs_per_row, by
+// multiplication (exact for l < 2^16).
 constexpr int kFlatRows = 64;
 constexpr int kFlatItems = 4;  // packs of a thread in flight together
 
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void mean_grad_flat_kernel(GatherArgs<T> a, int ppr, uint32_t magic) {
-    const int64_t row0 = (int64_t)blockIdx.x * kFlatRows;
-    const int rows = (int)min((int64_t)kFlatRows, a.N - row0);
+template <typename T, int VEC, int OP>
+__global__ __launch_bounds__(kBlock) void gather_flat_kernel(GatherArgs<T> a, int ppr, uint32_t magic,
+                                                             int rows_per_group) {
+    const int64_t row0 = (int64_t)blockIdx.x * rows_per_group;
+    const int rows = (int)min((int64_t)rows_per_group, a.N - row0);
     const int packs = rows * ppr;
     const LPack<T, VEC> *src = reinterpret_cast<const LPack<T, VEC> *>(a.src);
     T *out = a.out + row0 * a.F;
@@ -905,15 +907,26 @@ __global__ __launch_bounds__(kBlock) void mean_grad_flat_kernel(GatherArgs<T> a,
                 g[u] = g[u] < 0 ? 0 : a.groups - 1;
                 if (a.bad_id) *a.bad_id = 1;  // every writer stores the same value
             }
-            denom[u] = (T)max(a.counts[g[u]], 1);
+            if constexpr (OP == GATHER_MEAN_GRAD) denom[u] = (T)max(a.counts[g[u]], 1);
             x[u] = src[g[u] * ppr + col[u]];
         }
 #pragma unroll
         for (int u = 0; u < kFlatItems; ++u) {
             const int l = l0 + u * kBlock;
             if (l >= packs) break;
+            if constexpr (OP == GATHER_MEAN_GRAD) {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) x[u].v[i] = x[u].v[i] / denom[u];
+                for (int i = 0; i < VEC; ++i) x[u].v[i] = x[u].v[i] / denom[u];
+            } else {
+                LPack<T, VEC> b;
+                if (a.bias) b = reinterpret_cast<const LPack<T, VEC> *>(a.bias)[col[u]];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    T v = x[u].v[i];
+                    if (a.bias) v = v + b.v[i];
+                    x[u].v[i] = (a.relu && v < T(0)) ? T(0) : v;
+                }
+            }
             store_stream<T, VEC>(out + (int64_t)l * VEC, x[u]);
         }
     }
@@ -945,17 +958,15 @@ int launch_gather(const GatherArgs<T> &a, hipStream_t stream) {
     constexpr int WIDE = 16 / sizeof(T);
     auto al = [](const void *p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     const bool wide = a.F % WIDE == 0 && al(a.src) && al(a.out) && al(a.bias);
-    if constexpr (OP == GATHER_MEAN_GRAD) {
-        const int64_t ppr = a.F / WIDE;
-        if (wide && a.perm == nullptr && (a.F * (int64_t)sizeof(T)) % 128 != 0 && kFlatRows * ppr < (1 << 16) &&
-            ceil_div(a.N, kFlatRows) < ((int64_t)1 << 31)) {
-            const uint32_t magic = ppr > 1 ? (uint32_t)((1ull << 32) / (uint32_t)ppr) + 1u : 0u;
-            if (ppr > 1) {
-                hipLaunchKernelGGL((mean_grad_flat_kernel<T, WIDE>), dim3((unsigned)ceil_div(a.N, kFlatRows)), dim3(kBlock),
-                                   0, stream, a, (int)ppr, magic);
-                return check_launch("mean_grad_flat");
-            }
-        }
+    const int64_t ppr = a.F / WIDE;
+    if (wide && a.perm == nullptr && a.signs == nullptr && (a.F * (int64_t)sizeof(T)) % 128 != 0 && ppr > 1 &&
+        kFlatRows * ppr < (1 << 16) && ceil_div(a.N, kFlatRows) < ((int64_t)1 << 31)) {
+        const uint32_t magic = (uint32_t)((1ull << 32) / (uint32_t)ppr) + 1u;
+        // 64 rows, or as many times 64 as give the threads their four packs each
+        const int rows = kFlatRows * (int)std::max<int64_t>(1, kFlatItems * kBlock / (kFlatRows * ppr));
+        hipLaunchKernelGGL((gather_flat_kernel<T, WIDE, OP>), dim3((unsigned)ceil_div(a.N, rows)), dim3(kBlock), 0,
+                           stream, a, (int)ppr, magic, rows);
+        return check_launch("gather_flat");
     }
     if (wide) return launch_gather_lpr<T, WIDE, OP>(a, stream);
     return launch_gather_lpr<T, 1, OP>(a, stream);
