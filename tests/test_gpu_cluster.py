@@ -129,6 +129,29 @@ def test_assign_many_tiles_a_wave(width, bits):
     assert np.array_equal(counts.cpu().numpy(), want_counts)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("width", [8, 12, 16, 20, 36, 100, 132])
+@pytest.mark.parametrize("n", [63, 64, 65, 1025, 20011])
+def test_gathers_over_rows_that_are_not_whole_lines(dtype, width, n):
+    """Mean gradient and reconstruct in natural row order at widths whose rows are 16-byte
+    packs but not whole 128-byte lines: the output is then produced pack by pack, 64 rows or
+    a multiple of 64 a workgroup; row counts on both sides of those bounds, bit for bit
+    against the oracle."""
+    rng = np.random.default_rng(width * 100003 + n)
+    groups = 1 + min(n, 97)
+    ids_np = rng.integers(1, groups, size=n).astype(np.int64) if groups > 1 else np.zeros(n, np.int64)
+    counts_np = np.bincount(ids_np, minlength=groups).astype(np.int32)
+    ids, counts = torch.from_numpy(ids_np).to(DEV), torch.from_numpy(counts_np).to(DEV)
+    grad = rng.standard_normal((groups, width)).astype(dtype)
+    want_dx = oracle.cluster_mean_backward(grad, ids_np, counts_np)
+    assert np.array_equal(abi.cluster_mean_backward(_t(grad), ids, counts).cpu().numpy(), want_dx)
+    bias = rng.standard_normal(width).astype(dtype)
+    for relu in (False, True):
+        for b in (None, bias):
+            out = abi.reconstruct(_t(grad), ids, None if b is None else _t(b), relu)
+            assert np.array_equal(out.cpu().numpy(), oracle.reconstruct(grad, ids_np, b, relu))
+
+
 @pytest.mark.parametrize("shape", ["uniform", "one_code", "few_codes", "relu"])
 @pytest.mark.parametrize("bits", [1, 8, 16, 23])
 def test_grouped_assign_matches_counter_path(shape, bits):
